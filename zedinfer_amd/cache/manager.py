@@ -7,7 +7,8 @@ each request its own block table per group; all caches of a group share the
 page ids, so one table serves every layer of the group (the reference keeps a
 page list per layer, reference: src/backend/kvcache/block_pool.hpp:73-103).
 Pages go back to the pool when the request ends, or, in a window group, as soon
-as no later token can see them.  A page holds ``page_size`` tokens of one layer,
+as no later token can see them (a window group may also keep the pages of a
+sequence's first positions for good: ``KVCacheRequest.keep_first``).  A page holds ``page_size`` tokens of one layer,
 in the tensors the layer's mixer asked for (``KVCacheRequest.tensors``: names,
 shapes of one page, types): the manager allocates them and hands them over by
 name and knows nothing of what they hold (the reference's page is keys and values
@@ -34,6 +35,15 @@ from ..parts.base import KVCacheRequest, LayerMemory, StateRequest
 from .pages import IdPool, OutOfPages, PagePool
 
 
+EMBEDDING_CACHE = -1      # the id under which the embedding's state per request (if it keeps any) is asked for
+
+
+class Memories(list):
+    """The ``LayerMemory`` of every schedule step, and the embedding's."""
+
+    embedding: Optional[LayerMemory] = None
+
+
 @dataclass
 class CacheGroup:
     kind: str                      # "full" or "window"
@@ -41,6 +51,12 @@ class CacheGroup:
     page_size: int
     pool: PagePool
     caches: Dict[int, KVCacheRequest] = field(default_factory=dict)    # cache id -> what its layer asked for
+    keep_first: int = 0            # a window group keeps the pages of positions below this as well
+
+    @property
+    def kept_pages(self) -> int:
+        """Logical pages at the start of a sequence that a window group never gives back early."""
+        return self.pages_for(self.keep_first) if self.kind == "window" else 0
 
     def pages_for(self, tokens: int) -> int:
         return (tokens + self.page_size - 1) // self.page_size
@@ -49,7 +65,7 @@ class CacheGroup:
         """Most pages a sequence of ``tokens`` tokens holds at once in this group."""
         n = self.pages_for(tokens)
         if self.kind == "window":
-            n = min(n, self.pages_for(self.window - 1 + max(max_step_tokens, 1)) + 1)
+            n = min(n, self.pages_for(self.window - 1 + max(max_step_tokens, 1)) + 1 + self.kept_pages)
         return n
 
     def first_live_page(self, length: int) -> int:
@@ -100,15 +116,18 @@ class CacheManager:
         self.device = torch.device(device) if device is not None else None
         self.groups: List[CacheGroup] = []
         self.group_of_cache: Dict[int, int] = {}
-        keys: Dict[Tuple[str, int], int] = {}
+        keys: Dict[Tuple[str, int, int], int] = {}
         for cid in sorted(kv_requests):
             rq = kv_requests[cid]
             if rq.kind not in ("full", "window") or (rq.kind == "window" and rq.window <= 0):
                 raise ValueError(f"cache {cid}: unknown cache kind {rq.kind!r} / window {rq.window}")
-            key = (rq.kind, rq.window if rq.kind == "window" else 0)
+            if rq.keep_first < 0:
+                raise ValueError(f"cache {cid}: negative keep_first")
+            key = (rq.kind, rq.window if rq.kind == "window" else 0, rq.keep_first if rq.kind == "window" else 0)
             if key not in keys:
                 keys[key] = len(self.groups)
-                self.groups.append(CacheGroup(rq.kind, key[1], self.page_size, PagePool(self.num_pages)))
+                self.groups.append(CacheGroup(rq.kind, key[1], self.page_size, PagePool(self.num_pages),
+                                              keep_first=key[2]))
             g = keys[key]
             self.groups[g].caches[cid] = rq
             self.group_of_cache[cid] = g
@@ -139,8 +158,11 @@ class CacheManager:
                 total += n * torch.empty((), dtype=pt.dtype or dtype).element_size()
         return total
 
-    def memories(self, schedule: Sequence[ScheduleStep]) -> List[LayerMemory]:
-        out = []
+    def memories(self, schedule: Sequence[ScheduleStep]) -> "Memories":
+        """What every run of the schedule is bound to, in its order; ``embedding`` is what the embedding is (the
+        state that was asked for under EMBEDDING_CACHE)."""
+        out = Memories()
+        out.embedding = LayerMemory(state=self.state.get(EMBEDDING_CACHE))
         for st in schedule:
             g = self.group_of_cache.get(st.cache, -1)
             out.append(LayerMemory(group=g, tensors=self.tensors.get(st.cache, {}), writes=st.writes_cache,
@@ -180,7 +202,7 @@ class CacheManager:
                 continue
             first = min(g.first_live_page(seq.length), len(seq.pages[gi]))
             table = seq.pages[gi]
-            for i in range(first):
+            for i in range(g.kept_pages, first):
                 if table[i] >= 0:
                     g.pool.give_back(table[i])
                     table[i] = -1

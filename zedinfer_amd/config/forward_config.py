@@ -12,7 +12,7 @@ mixers and feed-forwards.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, Tuple
+from typing import Any, Dict, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -48,12 +48,15 @@ class ScheduleStep:
     than once).  ``cache`` names the cache/state buffer this run uses; two
     steps with the same ``cache`` share it.  Only a step with ``writes_cache``
     stores keys and values; a step that reads another step's cache sets it to
-    False and names that step's ``cache``.
+    False and names that step's ``cache``.  ``enter`` names a registered stream step (a ``PartSpec``) that is applied
+    to the residual stream right before the layer runs (what a design does to the stream between layers: adding the
+    embedding output again at the start of a repeated run of layers, for instance).
     """
 
     layer: int
     cache: int
     writes_cache: bool = True
+    enter: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)
@@ -75,6 +78,8 @@ class ModelForwardConfig:
     # flags on its forward config: forward_config.hpp:36-37).  Nothing in the engine reads it: what a part needs
     # is in its PartSpec.
     family: Dict[str, Any] = field(default_factory=dict)
+    # tensors a checkpoint may hold without the model reading them (the loader names every other stranger)
+    ignorable_tensors: Tuple[str, ...] = ()
 
     def validate(self) -> None:
         n = len(self.layers)

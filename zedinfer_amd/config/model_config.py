@@ -389,3 +389,120 @@ class TosisunConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+@dataclass(frozen=True)
+class TilivikConfig(ModelConfig):
+    """The Tilivik design's config.json: ``width``, ``vocab``, ``norm.eps``, ``embedding.bigram`` (``buckets``,
+    ``mul_prev``, ``mul_cur``; optional), ``loop`` (``start``, ``stop``, ``times``: layers start .. stop-1 run
+    ``times`` times in a row; optional) and a list ``layers`` whose entries each name a mixer by ``type``
+    ("lightning": linear attention with a fixed decay per head; "parallel": windowed softmax attention with a bias
+    by distance beside gated linear attention) with its sizes under ``mixer`` and a feed-forward under ``mlp``
+    (``kind`` "moe": experts named by a table of token ids; or null for none).  Every size and constant of a model is
+    read from here (the rows of a layer's bias table are the tensor's own unless ``mixer.left.bias_rows`` names
+    them); the shared keys of ``ModelConfig`` that the format does not have keep their neutral values."""
+
+    layers: Tuple[Any, ...] = ()
+    norm_eps: float = 1e-6
+    bigram: Any = None          # {"buckets", "mul_prev", "mul_cur"} or None
+    loop: Any = None            # {"start", "stop", "times"} or None
+
+    MIXER_KEYS = {"lightning": ("heads", "dim", "vdim", "decay"),
+                  "parallel": ("left", "right", "left_scale", "right_scale")}
+    LEFT_KEYS = ("heads", "kv_heads", "dim", "vdim", "scale")
+    RIGHT_KEYS = ("heads", "dim", "vdim", "tau")
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "TilivikConfig":
+        missing = [k for k in ("width", "vocab", "layers", "norm") if k not in d]
+        if missing:
+            raise ConfigError("config.json lacks required key(s): " + ", ".join(missing))
+        if not isinstance(d["layers"], (list, tuple)) or not d["layers"]:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        if not isinstance(d["norm"], Mapping) or "eps" not in d["norm"]:
+            raise ConfigError("config.json: 'norm' must give 'eps'")
+        eos = d.get("eos_token_id")
+        bigram = (d.get("embedding") or {}).get("bigram")
+        loop = d.get("loop")
+        cfg = cls(architectures=(str(d.get("architecture", "Tilivik")),), model_type="tilivik",
+                  torch_dtype=str(d.get("torch_dtype") or "bfloat16"), hidden_size=_as_int(d, "width"),
+                  vocab_size=_as_int(d, "vocab"), num_hidden_layers=len(d["layers"]),
+                  eos_token_ids=() if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos])),
+                  layers=tuple(json.loads(json.dumps(layer)) for layer in d["layers"]), norm_eps=float(d["norm"]["eps"]),
+                  bigram=json.loads(json.dumps(bigram)) if bigram else None,
+                  loop=json.loads(json.dumps(loop)) if loop else None)
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.hidden_size <= 0 or self.vocab_size <= 0:
+            raise ConfigError("config.json: 'width' and 'vocab' must be positive")
+        if not (self.norm_eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.norm_eps}")
+        if self.bigram is not None:
+            lacking = [k for k in ("buckets", "mul_prev", "mul_cur") if not isinstance(self.bigram, Mapping) or k not in self.bigram]
+            if lacking or int(self.bigram["buckets"]) <= 0:
+                raise ConfigError("config.json: embedding.bigram needs a positive 'buckets', 'mul_prev' and 'mul_cur'")
+        if self.loop is not None:
+            lp = self.loop
+            if not isinstance(lp, Mapping) or any(k not in lp for k in ("start", "stop", "times")) \
+                    or not (0 <= int(lp["start"]) < int(lp["stop"]) <= len(self.layers)) or int(lp["times"]) < 1:
+                raise ConfigError("config.json: loop needs 0 <= start < stop <= the number of layers and times >= 1")
+        for i, layer in enumerate(self.layers):
+            kind = layer.get("type") if isinstance(layer, Mapping) else None
+            if kind not in self.MIXER_KEYS:
+                raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
+            m = layer.get("mixer")
+            lacking = [k for k in self.MIXER_KEYS[kind] if not isinstance(m, Mapping) or k not in m]
+            if lacking:
+                raise ConfigError(f"config.json: layer {i} ({kind}) lacks mixer key(s): " + ", ".join(lacking))
+            if kind == "lightning":
+                if any(int(m[k]) <= 0 for k in ("heads", "dim", "vdim")) or len(m["decay"]) != int(m["heads"]):
+                    raise ConfigError(f"config.json: layer {i}: heads, dim and vdim must be positive, one decay a head")
+            else:
+                for side, keys in (("left", self.LEFT_KEYS), ("right", self.RIGHT_KEYS)):
+                    lacking = [k for k in keys if not isinstance(m[side], Mapping) or k not in m[side]]
+                    if lacking:
+                        raise ConfigError(f"config.json: layer {i}: mixer.{side} lacks key(s): " + ", ".join(lacking))
+                left, right = m["left"], m["right"]
+                if any(int(left[k]) <= 0 for k in ("heads", "kv_heads", "dim", "vdim")) or int(left["heads"]) % int(left["kv_heads"]):
+                    raise ConfigError(f"config.json: layer {i}: mixer.left: sizes must be positive, heads a multiple of kv_heads")
+                if not float(left["scale"]) > 0 or float(left.get("softcap") or 0) < 0:
+                    raise ConfigError(f"config.json: layer {i}: mixer.left: scale must be positive, softcap not negative")
+                mask = left.get("mask")
+                if mask is not None and (not int(mask.get("size", 0)) > 0 or int(mask.get("keep_first", 0)) < 0):
+                    raise ConfigError(f"config.json: layer {i}: mask.size must be positive, mask.keep_first not negative")
+                if any(int(right[k]) <= 0 for k in ("heads", "dim", "vdim")) or not float(right["tau"]) > 0:
+                    raise ConfigError(f"config.json: layer {i}: mixer.right: sizes and tau must be positive")
+            mlp = layer.get("mlp")
+            if mlp is None:
+                continue
+            if mlp.get("kind") != "moe":
+                raise ConfigError(f"config.json: layer {i}: mlp.kind {mlp.get('kind')!r} is not 'moe'")
+            r = mlp.get("router") or {}
+            if not int((mlp.get("expert") or {}).get("ff", 0)) > 0 or not (0 < int(r.get("top", 0)) <= int(r.get("experts", 0))):
+                raise ConfigError(f"config.json: layer {i}: a moe mlp needs expert.ff, router.experts and router.top "
+                                  "(at most the experts)")
+
+    def run_order(self):
+        """(layer, pass) in the order the layers run; pass is None outside the repeated run."""
+        L = len(self.layers)
+        if self.loop is None:
+            return [(i, None) for i in range(L)]
+        a, b, times = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        order = [(i, None) for i in range(a)]
+        for t in range(times):
+            order += [(i, t) for i in range(a, b)]
+        return order + [(i, None) for i in range(b, L)]
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"architecture": self.architectures[0] if self.architectures else "Tilivik",
+             "layers": json.loads(json.dumps(list(self.layers))), "norm": {"eps": self.norm_eps},
+             "vocab": self.vocab_size, "width": self.hidden_size}
+        if self.bigram is not None:
+            d["embedding"] = {"bigram": dict(self.bigram)}
+        if self.loop is not None:
+            d["loop"] = dict(self.loop)
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

@@ -9,6 +9,11 @@
 // src/backend/ops/self_attention/cpu/paged_attention_cpu.cpp:106-162; the scale
 // after the dot product at :135, the causal bound at :116).
 //
+// Optional, for mixers that have them: a smooth cap of the scaled score (cap * tanh(s / cap)), a learned bias
+// added after it, looked up by the distance p - j in a table [heads][bias_len] (distances beyond the table take
+// its last entry), and, beside a window, the first `keep_first` positions of the sequence, which stay visible at
+// their true distances when the window has passed them.
+//
 // It takes every head size up to 512, any number of heads and groups, any page
 // size, both storage types, prompts and decoded tokens alike, and its result
 // for a token depends only on that token's position and keys, not on the
@@ -27,7 +32,8 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
                          const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                          int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
-                         float scale, const float* __restrict__ sinks) {
+                         float scale, const float* __restrict__ sinks, float softcap,
+                         const float* __restrict__ bias, int bias_len, int keep_first) {
     __shared__ float qs[ATTN_MAX_D];
     __shared__ float ps[ZI_WAVE];
     __shared__ int64_t vbase[ZI_WAVE];
@@ -36,6 +42,10 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
     const int p = tok_pos[t];
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    // the keys a token sees, in rising order: the kept first positions that the window has passed, then [lo, p]
+    const int kept = keep_first < lo ? (keep_first > 0 ? keep_first : 0) : lo;
+    const int count = kept + (p - lo + 1);
+    const float* brow = bias ? bias + (int64_t)h * bias_len : nullptr;
 
     const T* qr = q + (int64_t)t * ldq + (int64_t)h * d;
     for (int j = lane; j < d; j += ZI_WAVE) qs[j] = zi_load(qr + j);
@@ -46,9 +56,10 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
 #pragma unroll
     for (int i = 0; i < ATTN_ACC; ++i) acc[i] = 0.f;
 
-    for (int base = lo; base <= p; base += ZI_WAVE) {
-        const int j = base + lane;
-        bool valid = j <= p;
+    for (int base = 0; base < count; base += ZI_WAVE) {
+        const int at = base + lane;
+        bool valid = at < count;
+        const int j = at < kept ? at : lo + (at - kept);
         float s = -INFINITY;
         int64_t row = -1, vrow = -1;
         if (valid) {
@@ -63,6 +74,8 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
                 float dot = 0.f;
                 for (int x = 0; x < d; ++x) dot += qs[x] * zi_load(kr + x);
                 s = dot * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+                if (brow) s += brow[p - j < bias_len ? p - j : bias_len - 1];
             }
         }
         const float mt = zi_wave_max(s);
@@ -73,7 +86,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
         ps[lane] = pj;
         vbase[lane] = vrow;
         __syncthreads();
-        const int cnt = (p - base + 1 < ZI_WAVE) ? p - base + 1 : ZI_WAVE;
+        const int cnt = (count - base < ZI_WAVE) ? count - base : ZI_WAVE;
 #pragma unroll
         for (int i = 0; i < ATTN_ACC; ++i) acc[i] *= corr;
         for (int jj = 0; jj < cnt; ++jj) {
@@ -100,12 +113,16 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
     }
 }
 
-// `sinks` (float32 [nh], or null): the softmax of head h also counts exp(sinks[h]) in its denominator.
-extern "C" int zi_attention_generic_sink(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
+// `sinks` (float32 [nh], or null): the softmax of head h also counts exp(sinks[h]) in its denominator.  `softcap` > 0
+// caps the scaled scores; `bias` (float32 [nh][bias_len], or null) is added by distance; `keep_first` positions stay
+// visible beside the window.
+extern "C" int zi_attention_generic_biased(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
                                          const void* kcache, const void* vcache, const int32_t* tok_index,
                                          const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
                                          int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
-                                         float scale, const float* sinks, hipStream_t stream) {
+                                         float scale, const float* sinks, float softcap, const float* bias,
+                                         int bias_len, int keep_first, hipStream_t stream) {
+    ZI_REQUIRE(softcap >= 0.f && keep_first >= 0 && (!bias || bias_len > 0), "attention: bad cap, bias or kept positions");
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0 && max_pages > 0 && num_pages > 0,
                "attention: bad sizes");
     ZI_REQUIRE(nh % nkv == 0, "attention: %d query heads are not a multiple of %d key/value heads", nh, nkv);
@@ -117,9 +134,19 @@ extern "C" int zi_attention_generic_sink(void* out, const void* q, int dt, int n
     ZI_DISPATCH_DTYPE(dt, T, {
         attention_generic_kernel<T><<<dim3(n, nh), ZI_WAVE, 0, stream>>>(
             (T*)out, (const T*)q, ldq, ldo, (const T*)kcache, (const T*)vcache, tok_index, tok_seq, tok_pos, block_tables,
-            max_pages, num_pages, nh, nkv, d, page_size, window, scale, sinks);
+            max_pages, num_pages, nh, nkv, d, page_size, window, scale, sinks, softcap, bias, bias_len, keep_first);
     });
     return zi_check_launch("attention_generic");
+}
+
+extern "C" int zi_attention_generic_sink(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
+                                         const void* kcache, const void* vcache, const int32_t* tok_index,
+                                         const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                         int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                                         float scale, const float* sinks, hipStream_t stream) {
+    return zi_attention_generic_biased(out, q, dt, n, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos, block_tables,
+                                       max_pages, num_pages, nh, nkv, d, page_size, window, scale, sinks, 0.f, nullptr, 0,
+                                       0, stream);
 }
 
 extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,

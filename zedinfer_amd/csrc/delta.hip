@@ -311,11 +311,13 @@ extern "C" int zi_delta_rule(float* out, const float* qk, const float* v, const 
 }
 
 // o [rows][vdim] (a row per token and head) divided by its root mean square, times a weight [vdim], times
-// SiLU of a gate read from gate[token][head * vdim + e] with row stride ld_gate.  A wavefront per row.
+// an activation of a gate read from gate[token][head * vdim + e] with row stride ld_gate (act 0: SiLU, 1: sigmoid),
+// times `scale`; the result goes to out[token][head * vdim + e] with row stride ldo.  A wavefront per row.
 template <typename TO, typename TW>
 __global__ void __launch_bounds__(256)
-gated_rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ o, const TW* __restrict__ w,
-                     const float* __restrict__ gate, int64_t ld_gate, int rows, int heads, int vdim, float eps) {
+gated_rmsnorm_kernel(TO* __restrict__ out, int64_t ldo, const float* __restrict__ o, const TW* __restrict__ w,
+                     const float* __restrict__ gate, int64_t ld_gate, int rows, int heads, int vdim, float eps, int act,
+                     float scale) {
     const int lane = threadIdx.x % ZI_WAVE;
     const int64_t row = (int64_t)blockIdx.x * (blockDim.x / ZI_WAVE) + threadIdx.x / ZI_WAVE;
     if (row >= rows) return;
@@ -325,18 +327,31 @@ gated_rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ o, const TW
     ss = zi_wave_sum(ss);
     const float rstd = 1.f / sqrtf(ss / (float)vdim + eps);
     const float* grow = gate + (row / heads) * ld_gate + (row % heads) * vdim;
-    for (int j = lane; j < vdim; j += ZI_WAVE)
-        zi_store(out + row * vdim + j, orow[j] * rstd * zi_load(w + j) * delta_silu(grow[j]));
+    TO* dst = out + (row / heads) * ldo + (row % heads) * vdim;
+    for (int j = lane; j < vdim; j += ZI_WAVE) {
+        const float g = grow[j];
+        const float a = act == 1 ? 1.f / (1.f + expf(-g)) : delta_silu(g);
+        zi_store(dst + j, orow[j] * rstd * zi_load(w + j) * a * scale);
+    }
+}
+
+extern "C" int zi_gated_rmsnorm_act(void* out, int out_dt, int64_t ldo, const float* o, const void* w, int w_dt,
+                                    const float* gate, int64_t ld_gate, int n, int heads, int vdim, float eps, int act,
+                                    float scale, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && heads > 0 && vdim > 0 && eps > 0.f && ld_gate >= (int64_t)heads * vdim &&
+               ldo >= (int64_t)heads * vdim, "gated_rmsnorm: bad sizes");
+    ZI_REQUIRE(act == 0 || act == 1, "gated_rmsnorm: unknown gate activation %d", act);
+    if (n == 0) return 0;
+    const int rows = n * heads;
+    ZI_DISPATCH_DTYPE(out_dt, TO, ZI_DISPATCH_DTYPE(w_dt, TW, {
+        gated_rmsnorm_kernel<TO, TW><<<(rows + 3) / 4, 256, 0, stream>>>((TO*)out, ldo, o, (const TW*)w, gate, ld_gate,
+                                                                         rows, heads, vdim, eps, act, scale);
+    }));
+    return zi_check_launch("gated_rmsnorm");
 }
 
 extern "C" int zi_gated_rmsnorm(void* out, int out_dt, const float* o, const void* w, int w_dt, const float* gate,
                                 int64_t ld_gate, int n, int heads, int vdim, float eps, hipStream_t stream) {
-    ZI_REQUIRE(n >= 0 && heads > 0 && vdim > 0 && eps > 0.f && ld_gate >= (int64_t)heads * vdim, "gated_rmsnorm: bad sizes");
-    if (n == 0) return 0;
-    const int rows = n * heads;
-    ZI_DISPATCH_DTYPE(out_dt, TO, ZI_DISPATCH_DTYPE(w_dt, TW, {
-        gated_rmsnorm_kernel<TO, TW><<<(rows + 3) / 4, 256, 0, stream>>>((TO*)out, o, (const TW*)w, gate, ld_gate, rows,
-                                                                         heads, vdim, eps);
-    }));
-    return zi_check_launch("gated_rmsnorm");
+    return zi_gated_rmsnorm_act(out, out_dt, (int64_t)heads * vdim, o, w, w_dt, gate, ld_gate, n, heads, vdim, eps, 0, 1.f,
+                                stream);
 }

@@ -3,6 +3,7 @@
 //
 //   zi_moe_route    z [n][E] float32 router logits -> s = softmax(z); choice = s + correction; the `top` experts
 //                   of largest choice (the lowest index among equals), weights s * scale
+//   zi_moe_route_table  the experts of a token are read from a table by its id, equal weights
 //   zi_moe_group    the (token, choice) pairs sorted by expert: offsets, the order and its inverse, and the list
 //                   of row tiles (expert, first row, rows) that the products walk
 //   zi_moe_linear   out[row] = act(W[expert of row] . x[source of row]) for every row of the sorted order
@@ -156,6 +157,31 @@ extern "C" int zi_moe_route_top(int32_t* idx, float* wt, const float* z, const f
     else ZI_MOE_ROUTE(MOE_PER_LANE);
 #undef ZI_MOE_ROUTE
     return zi_check_launch("moe_route_top");
+}
+
+// Experts named by a table instead of a router: token id v uses the experts table[v][0 .. top), each with the
+// weight 1 / top.  An id outside the table, or an entry that names no expert, gives expert 0 with weight NaN so
+// that the fault shows.
+__global__ void __launch_bounds__(256)
+moe_route_table_kernel(int32_t* __restrict__ idx, float* __restrict__ wt, const int32_t* __restrict__ ids,
+                       const int32_t* __restrict__ table, int pairs, int vocab, int E, int top) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= pairs) return;
+    const int id = ids[i / top];
+    const int e = (id >= 0 && id < vocab) ? table[(int64_t)id * top + i % top] : -1;
+    const bool ok = e >= 0 && e < E;
+    idx[i] = ok ? e : 0;
+    wt[i] = ok ? 1.f / (float)top : NAN;
+}
+
+extern "C" int zi_moe_route_table(int32_t* idx, float* wt, const int32_t* ids, const int32_t* table, int n, int vocab,
+                                  int experts, int top, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && vocab > 0 && experts > 0 && experts <= MOE_MAX_EXPERTS && top > 0 && top <= experts,
+               "moe_route_table: bad sizes (experts %d, top %d; at most %d experts)", experts, top, MOE_MAX_EXPERTS);
+    if (n == 0) return 0;
+    const int pairs = n * top;
+    moe_route_table_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>(idx, wt, ids, table, pairs, vocab, experts, top);
+    return zi_check_launch("moe_route_table");
 }
 
 // One workgroup sorts the M = n * top pairs by expert (a counting sort; within an expert the order is the order

@@ -198,6 +198,44 @@ int zi_moe_route_top(int32_t* idx, float* wt, const float* z, const float* bias,
 // sampling.hip
 int zi_argmax(int32_t* out_idx, float* out_val, const void* logits, int dt, int rows, int vocab, int64_t ld, float*
     workspace, int64_t workspace_floats, hipStream_t stream);
+// stream.hip
+int zi_embedding_sum(float* out, const void* table, int table_dt, const void* pair, int pair_dt, const int32_t* ids,
+    const int32_t* pos, const int32_t* tok_seq, const int32_t* entry_start, const int32_t* entry_len, const int32_t*
+    entry_slot, int32_t* state, int64_t state_stride, const double* freq, int n, int hidden, int vocab, int buckets,
+    int64_t mul_prev, int64_t mul_cur, hipStream_t stream);
+// stream.hip
+int zi_token_shift(void* out, int out_dt, int64_t ldo, const void* x, int x_dt, int64_t ldx, const void* w, int w_dt,
+    float* state, int64_t state_stride, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* entry_start,
+    const int32_t* entry_len, const int32_t* entry_slot, int n, int hidden, hipStream_t stream);
+// stream.hip
+int zi_stream_reenter(float* resid, const void* delta, int delta_dt, int splits, int64_t split_stride, const float*
+    again, const void* row, int row_dt, int n, int hidden, hipStream_t stream);
+// linear_attention.hip
+int zi_lowrank_decay(float* out, int64_t ldo, const float* u, int64_t ldu, const void* w2, const void* bias, int w_dt,
+    int n, int channels, int rank, float tau, hipStream_t stream);
+// linear_attention.hip
+int zi_linear_attention(float* out, int64_t ldo, const float* q, const float* k, const float* v, int64_t ld, const
+    float* decay, int64_t ld_decay, const float* head_decay, float* state, int64_t state_stride, const int32_t*
+    entry_start, const int32_t* entry_len, const int32_t* entry_past, const int32_t* entry_slot, int entries, int
+    heads, int dim, int vdim, int act, float qscale, hipStream_t stream);
+// linear_attention.hip
+int zi_gate_heads(void* out, int out_dt, int64_t ldo, const void* x, int x_dt, int64_t ldx, int x_head, const float*
+    gate, int64_t ld_gate, int n, int width, int head, int act, float scale, hipStream_t stream);
+// delta.hip
+int zi_gated_rmsnorm_act(void* out, int out_dt, int64_t ldo, const float* o, const void* w, int w_dt, const float*
+    gate, int64_t ld_gate, int n, int heads, int vdim, float eps, int act, float scale, hipStream_t stream);
+// attention_biased.hip
+int zi_normed_kv_store(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const float* proj, int64_t ld,
+    int q_at, int k_at, int v_at, const int32_t* slots, int64_t cache_slots, int n, int nh, int nkv, int dim, int vdim,
+    int d, int page_size, float eps, int norm_values, hipStream_t stream);
+// attention_generic.hip
+int zi_attention_generic_biased(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo, const void* kcache,
+    const void* vcache, const int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, const
+    float* sinks, float softcap, const float* bias, int bias_len, int keep_first, hipStream_t stream);
+// moe.hip
+int zi_moe_route_table(int32_t* idx, float* wt, const int32_t* ids, const int32_t* table, int n, int vocab, int
+    experts, int top, hipStream_t stream);
 // sampling.hip
 int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int rows, int vocab, const float*
     temperature, const int32_t* top_k, const float* top_p, const float* penalty, const float* uniform, const int32_t*
@@ -256,5 +294,15 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_softcap) \
     X(zi_convert) \
     X(zi_moe_route_top) \
+    X(zi_embedding_sum) \
+    X(zi_token_shift) \
+    X(zi_stream_reenter) \
+    X(zi_lowrank_decay) \
+    X(zi_linear_attention) \
+    X(zi_gate_heads) \
+    X(zi_gated_rmsnorm_act) \
+    X(zi_normed_kv_store) \
+    X(zi_attention_generic_biased) \
+    X(zi_moe_route_table) \
     X(zi_argmax) \
     X(zi_sample)

@@ -112,7 +112,7 @@ class Engine:
         arch, cfg = load_config(folder)
         fc = arch.forward_config(cfg)
         dt = parse_dtype(dtype)
-        weights = load_weights(folder, expected_weights(fc), dt, device)
+        weights = load_weights(folder, expected_weights(fc), dt, device, ignorable=fc.ignorable_tensors)
         engine = cls(fc, weights, dt, sched, device)
         engine.default_sampling = default_sampling(folder)
         return engine

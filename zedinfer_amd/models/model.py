@@ -13,8 +13,9 @@ import torch
 
 from .. import ops
 from ..config.forward_config import ModelForwardConfig, PartSpec
-from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, KVCacheRequest, LayerMemory, Part,
-                     Runtime, StateRequest)
+from ..cache.manager import EMBEDDING_CACHE
+from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, STREAM_STEPS, KVCacheRequest, LayerMemory,
+                     Part, Runtime, StateRequest)
 from ..weights.loader import WeightSpec
 
 
@@ -46,6 +47,9 @@ def expected_weights(fc: ModelForwardConfig) -> Dict[str, WeightSpec]:
         merge(_part_weights(FEED_FORWARDS, layer.feed_forward))
         for n in layer.norms.values():
             merge(_part_weights(NORMS, n))
+    for st in fc.schedule:
+        if st.enter is not None:
+            merge(_part_weights(STREAM_STEPS, st.enter))
     merge(_part_weights(NORMS, fc.final_norm))
     merge(_part_weights(HEADS, fc.lm_head))
     return exp
@@ -77,6 +81,10 @@ class DecoderModel:
             # a mixer's position encoding is a part of its own
             self.parts += [self.blocks[-1], mixer, ffn, *norms.values()]
             self.parts += [p for p in vars(mixer).values() if isinstance(p, Part)]
+        # what a schedule step does to the stream before its layer runs
+        self.enters = [(_build(STREAM_STEPS, st.enter, weights, rt) if st.enter is not None else None) for st in fc.schedule]
+        self.parts += [e for e in self.enters if e is not None]
+        self.keeps_embedded = any(getattr(e, "needs_embedded", False) for e in self.enters if e is not None)
         self.final_norm = _build(NORMS, fc.final_norm, weights, rt)
         self.lm_head = _build(HEADS, fc.lm_head, weights, rt)
         self.parts += [self.embedding, self.final_norm, self.lm_head]
@@ -109,7 +117,13 @@ class DecoderModel:
         return out
 
     def state_requests(self) -> Dict[int, StateRequest]:
+        """cache id -> the state per request that the mixer of the step asks for; what the embedding asks for (the
+        token before, in a design whose embedding reads it) stands under EMBEDDING_CACHE."""
         out: Dict[int, StateRequest] = {}
+        emb = getattr(self.embedding, "state_request", None)
+        req = emb() if emb is not None else None
+        if req is not None:
+            out[EMBEDDING_CACHE] = req
         for st in self.fc.schedule:
             req = self.blocks[st.layer].mixer.state_request()
             if req is not None:
@@ -149,8 +163,10 @@ class DecoderModel:
         return max([int(getattr(p, "position_axes", 1)) for p in self.parts] + [1])
 
     def padding_safe(self) -> bool:
-        """Whether steps may be padded to recurring shapes: every mixer says that padding is harmless to it."""
-        return all(getattr(b.mixer, "padding_safe", False) for b in self.blocks)
+        """Whether steps may be padded to recurring shapes: every mixer says that padding is harmless to it (and an
+        embedding that keeps state per request as well)."""
+        return all(getattr(b.mixer, "padding_safe", False) for b in self.blocks) and \
+            getattr(self.embedding, "padding_safe", True)
 
     def graph_safe(self) -> bool:
         """Whether a step's launches can be captured and replayed: every part says so."""
@@ -167,9 +183,17 @@ class DecoderModel:
         shared = getattr(batch, "shared", None)
         if shared is not None:
             shared.clear()      # what parts share holds for one run: a batch object may serve several steps
-        resid = self.embedding.forward(batch.token_ids)
+        if getattr(self.embedding, "reads_batch", False):
+            resid = self.embedding.forward(batch.token_ids, batch=batch, memory=getattr(memories, "embedding", None))
+        else:
+            resid = self.embedding.forward(batch.token_ids)
+        embedded = None
+        if self.keeps_embedded:
+            embedded = ops.convert(resid, self.rt.buffer("embedded", tuple(resid.shape), torch.float32))
         delta = None
-        for st, mem in zip(self.fc.schedule, memories):
+        for st, mem, enter in zip(self.fc.schedule, memories, self.enters):
+            if enter is not None:
+                delta = enter.forward(resid, delta, embedded)
             delta = self.blocks[st.layer].forward(resid, delta, batch, mem)
         if batch.num_logit_rows == 0:
             if delta is not None:

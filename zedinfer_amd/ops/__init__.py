@@ -24,6 +24,9 @@ from .mixing import (delta_conv_state, delta_prepare, delta_rule, delta_state_fl
                      moe_max_tiles, moe_route, moe_tile_rows, rope_pairs)
 from .sublayers import (clamped_glu, conv_qkv, conv_state_floats, conv_tail, convert, layer_norm, moe_route_top,
                         relu_squared, softcap)
+from .recurrent import (attention_biased, embedding_sum, gate_heads, gated_rms_norm_act, linear_attention,
+                        linear_attention_state_floats, lowrank_decay, moe_route_table, normed_kv_store, stream_reenter,
+                        token_shift)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
@@ -43,5 +46,7 @@ __all__ = [
     "moe_max_tiles", "moe_route", "moe_tile_rows", "rope_pairs",
     "clamped_glu", "conv_qkv", "conv_state_floats", "conv_tail", "convert", "layer_norm", "moe_route_top", "relu_squared",
     "softcap",
+    "attention_biased", "embedding_sum", "gate_heads", "gated_rms_norm_act", "linear_attention",
+    "linear_attention_state_floats", "lowrank_decay", "moe_route_table", "normed_kv_store", "stream_reenter", "token_shift",
     "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

@@ -98,6 +98,16 @@ _PROTOTYPES = {
     "zi_softcap": [P, L, F, P],
     "zi_convert": [P, I, P, I, L, P],
     "zi_moe_route_top": [P, P, P, P, I, I, I, P],
+    "zi_embedding_sum": [P, P, I, P, I, P, P, P, P, P, P, P, L, P, I, I, I, I, L, L, P],
+    "zi_token_shift": [P, I, L, P, I, L, P, I, P, L, P, P, P, P, P, I, I, P],
+    "zi_stream_reenter": [P, P, I, I, L, P, P, I, I, I, P],
+    "zi_lowrank_decay": [P, L, P, L, P, P, I, I, I, I, F, P],
+    "zi_linear_attention": [P, L, P, P, P, L, P, L, P, P, L, P, P, P, P, I, I, I, I, I, F, P],
+    "zi_gate_heads": [P, I, L, P, I, L, I, P, L, I, I, I, I, F, P],
+    "zi_gated_rmsnorm_act": [P, I, L, P, P, I, P, L, I, I, I, F, I, F, P],
+    "zi_normed_kv_store": [P, I, L, P, P, P, L, I, I, I, P, L, I, I, I, I, I, I, I, F, I, P],
+    "zi_attention_generic_biased": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, F, P, I, I, P],
+    "zi_moe_route_table": [P, P, P, P, I, I, I, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
     "zi_tape_record_many": [P, c_char_p, P, P, I],
     "zi_tape_run": [P, P],

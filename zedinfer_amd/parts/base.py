@@ -127,6 +127,7 @@ POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
+STREAM_STEPS = Registry("stream step")
 
 register_mixer = MIXERS.register
 register_feed_forward = FEED_FORWARDS.register
@@ -135,6 +136,7 @@ register_position_encoding = POSITION_ENCODINGS.register
 register_block = BLOCKS.register
 register_embedding = EMBEDDINGS.register
 register_head = HEADS.register
+register_stream_step = STREAM_STEPS.register
 
 
 PAGE = -1      # in the shape of a page tensor: where the number of tokens a page holds goes
@@ -155,13 +157,15 @@ class PageTensor:
 @dataclass(frozen=True)
 class KVCacheRequest:
     """What a mixer needs from the paged cache: pages for all positions ("full") or for the last ``window``
-    positions ("window"), and in every page the named ``tensors`` (name, PageTensor).  The cache manager
+    positions ("window"; with ``keep_first`` the pages of a sequence's first ``keep_first`` positions are kept as
+    well when the window has passed them), and in every page the named ``tensors`` (name, PageTensor).  The cache manager
     allocates [pages, *page shape] for each and hands them to the mixer's runs by name
     (``LayerMemory.tensors``); what they hold and how they are laid out is the mixer's business."""
 
     kind: str
     window: int = 0
     tensors: Tuple[Tuple[str, PageTensor], ...] = ()
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)
@@ -315,7 +319,10 @@ class Mixer(Part):
 
 class FeedForward(Part):
     """``forward(x)``: [n, hidden] -> [n, hidden] (or a stack [S, n, hidden] of float32 partial
-    sums, as for a mixer), token by token."""
+    sums, as for a mixer), token by token.  A feed-forward that needs more of the step than the rows (the token
+    ids, for one that picks experts by them) sets ``reads_batch`` and is called as ``forward(x, batch=batch)``."""
+
+    reads_batch: bool = False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -355,6 +362,19 @@ class PositionEncoding(Part):
         return None
 
     def encode(self, q, k, positions, nh: int, nkv: int, d: int) -> None:
+        raise NotImplementedError
+
+
+class StreamStep(Part):
+    """Something done to the residual stream between two layers, named by a step of the schedule
+    (``ScheduleStep.enter``): ``forward(resid, delta, embedded)`` gets the float32 stream [n, hidden], the addition
+    still pending from the layer before (or None; it must be folded in) and the embedding's output as it was
+    before the first layer (float32 [n, hidden]; kept only for models one of whose stream steps says
+    ``needs_embedded``), changes ``resid`` in place and returns the addition that is pending afterwards (None)."""
+
+    needs_embedded: bool = False
+
+    def forward(self, resid, delta, embedded):
         raise NotImplementedError
 
 

@@ -26,12 +26,17 @@ class PreNormBlock(Block):
         self.norm_post = norms["post_mixer"]
         self.mixer = mixer
         self.feed_forward = feed_forward
+        self.has_ff = getattr(feed_forward, "kind", "") != "none"      # without one the mixer's addition is handed on
         self.rt = rt
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, memory: LayerMemory):
         x = self.norm_in.add_forward(resid, delta) if delta is not None else self.norm_in.forward(resid)
         a = self.mixer.forward(x, batch, memory)
+        if not self.has_ff:
+            return a
         y = self.norm_post.add_forward(resid, a)
+        if self.feed_forward.reads_batch:
+            return self.feed_forward.forward(y, batch=batch)
         return self.feed_forward.forward(y)
 
 
@@ -73,6 +78,8 @@ class ParallelBlock(Block):
         terms = self.rt.buffer("parallel_terms", (2 if self.has_ff else 1, n, H), torch.float32)
         self._term(terms[0], self.mixer, x, batch, memory)
         if self.has_ff:
+            if self.feed_forward.reads_batch:
+                raise ValueError("the parallel block hands its feed-forward the rows alone")
             self._term(terms[1], self.feed_forward, x)
         return terms
 
@@ -116,7 +123,8 @@ class OutputNormBlock(Block):
         a = self.mixer.forward(x, batch, memory)
         x = self.norm_mixer.add_normed(resid, a)
         if self.has_ff:
-            f = self.feed_forward.forward(x if x is not None else resid)
+            kw = {"batch": batch} if self.feed_forward.reads_batch else {}
+            f = self.feed_forward.forward(x if x is not None else resid, **kw)
             x = self.norm_ff.add_normed(resid, f)
         shared = getattr(batch, "shared", None)
         if shared is not None:

@@ -454,3 +454,70 @@ class ClampedExperts(FeedForward):
             else:
                 ops.linear(act_s, self.shared.down, out=terms[1])
         return terms
+
+
+@register_feed_forward("table_experts")
+class TableExperts(FeedForward):
+    """A mixture of small gated feed-forwards down_e(act(gate_e x) * up_e x), no biases, without a router: an
+    integer table [vocab_size, top] names the experts of every token id (the entries of a row differ); each counts
+    1 / top, and the result is the weighted sum in float32.
+
+    Grouping, the experts' products and the sum are the routed mixtures' kernels (``csrc/moe.hip``); the table is
+    read on the device by the step's token ids, so the launches of a step do not depend on its tokens.
+    params: hidden_size, vocab_size, experts, top, ff, activation ("silu")."""
+
+    graph_safe = True
+    tape_safe = True
+    writes_into = True
+    reads_batch = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, V, E, top, ff = (int(p[k]) for k in ("hidden_size", "vocab_size", "experts", "top", "ff"))
+        w = {"table": WeightSpec((V, top), kind="int", high=E)}
+        for e in range(E):
+            w[f"gate_{e}"] = WeightSpec((ff, H))
+            w[f"up_{e}"] = WeightSpec((ff, H))
+            w[f"down_{e}"] = WeightSpec((H, ff))
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.experts, self.top, self.ff = int(p["hidden_size"]), int(p["experts"]), int(p["top"]), int(p["ff"])
+        self.activation = str(p.get("activation", "silu"))
+        if not (0 < self.top <= self.experts):
+            raise ValueError(f"table_experts: top {self.top} of {self.experts} experts")
+        self.table = weights["table"].to(torch.int32).contiguous()
+        E = self.experts
+        self.gate_up = torch.stack([torch.cat([weights[f"gate_{e}"], weights[f"up_{e}"].to(weights[f"gate_{e}"].dtype)])
+                                    for e in range(E)]).contiguous()
+        self.down = torch.stack([weights[f"down_{e}"] for e in range(E)]).contiguous()
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def forward(self, x: torch.Tensor, batch=None, out=None) -> torch.Tensor:
+        if batch is None:
+            raise ValueError("table_experts: the step's token ids are needed")
+        n, E, top, ff, rt = x.shape[0], self.experts, self.top, self.ff, self.rt
+        pairs = n * top
+        idx = rt.buffer("moe_choice", (n, top), torch.int32)
+        wt = rt.buffer("moe_weight", (n, top), torch.float32)
+        ops.moe_route_table(batch.token_ids, self.table, E, idx, wt)
+        rows = ops.moe_tile_rows(x.dtype, self.gate_up.dtype, (self.hidden, ff), pairs, E)
+        tiles = ops.moe_max_tiles(pairs, E, rows)
+        plan = rt.buffer("moe_plan", (1 + 3 * tiles,), torch.int32)
+        order = rt.buffer("moe_order", (pairs,), torch.int32)
+        place_of = rt.buffer("moe_place", (pairs,), torch.int32)
+        ops.moe_group(idx, E, rows, plan, order, place_of)
+        gu = rt.buffer("moe_gate_up", (pairs, 2 * ff), torch.float32)
+        ops.moe_linear(x, self.gate_up, plan, rows, tiles, out=gu, source=order, source_div=top)
+        act = rt.buffer("moe_act", (pairs, ff))
+        ops.gated_act(gu[:, :ff], gu[:, ff:], self.activation, out=act)
+        y = rt.buffer("moe_out_rows", (pairs, self.hidden), torch.float32)
+        ops.moe_linear(act, self.down, plan, rows, tiles, out=y)
+        if out is None:
+            out = rt.buffer("moe_out", (n, self.hidden), torch.float32)
+        return ops.moe_combine(y, wt, place_of, out)

@@ -15,7 +15,10 @@ from .base import Norm, Runtime, register_norm
 class RMSNorm(Norm):
     """y = w * x * rsqrt(mean(x^2) + eps); with ``add_one`` the weight is (1 + w)
     (reference: src/backend/ops/rms_norm/cpu/rms_norm_cpu.cpp:14-29).
-    params: dim, eps, add_one (default False)."""
+    With ``scalar`` the checkpoint holds ONE number (a tensor without axes) that multiplies every coordinate; it is
+    spread over ``dim`` values at load, so the kernels are the same.  ``out_dtype`` "float32": the normed rows leave
+    in float32 whatever the engine's activation type (for a reader that works on them in float32 before any product).
+    params: dim, eps, add_one (default False), scalar (False), out_dtype (None)."""
 
     graph_safe = True
     tape_safe = True
@@ -23,8 +26,8 @@ class RMSNorm(Norm):
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         # a gain: 1 in random-weights mode (0 when the norm multiplies by 1 + w)
-        return {"weight": WeightSpec((int(spec.params["dim"]),),
-                                     init="zeros" if spec.params.get("add_one", False) else "ones")}
+        shape = () if spec.params.get("scalar", False) else (int(spec.params["dim"]),)
+        return {"weight": WeightSpec(shape, init="zeros" if spec.params.get("add_one", False) else "ones")}
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)
@@ -32,14 +35,31 @@ class RMSNorm(Norm):
         self.eps = float(spec.params["eps"])
         self.add_one = bool(spec.params.get("add_one", False))
         self.weight = weights["weight"]
+        if spec.params.get("scalar", False):
+            self.weight = self.weight.reshape(1).expand(self.dim).contiguous()
+        self.out_dtype = torch.float32 if spec.params.get("out_dtype") == "float32" else None
 
     def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        out = self.rt.buffer("norm_out", (x.shape[0], self.dim), out_dtype or self.rt.dtype)
+        out = self.rt.buffer("norm_out", (x.shape[0], self.dim), out_dtype or self.out_dtype or self.rt.dtype)
         return ops.rms_norm(x, self.weight, self.eps, out=out, add_one=self.add_one)
 
     def add_forward(self, resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
-        out = self.rt.buffer("norm_out", (resid.shape[0], self.dim), self.rt.dtype)
+        out = self.rt.buffer("norm_out", (resid.shape[0], self.dim), self.out_dtype or self.rt.dtype)
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out=out, add_one=self.add_one)
+
+
+@register_norm("none")
+class NoNorm(Norm):
+    """Stands where a block arrangement names a norm that a layer does not have (the norm before a feed-forward
+    that is not there); it is never run."""
+
+    graph_safe = True
+    tape_safe = True
+
+    def forward(self, x, out_dtype=None):
+        raise ValueError("a layer without this norm was asked to run it")
+
+    add_forward = forward
 
 
 @register_norm("layernorm")

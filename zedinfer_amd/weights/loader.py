@@ -37,12 +37,14 @@ class WeightError(ValueError):
 class WeightSpec:
     """What a part needs from the checkpoint for one parameter."""
 
-    shape: Tuple[int, ...]
+    shape: Tuple[int, ...]           # -1: the checkpoint's own size on that axis
     kind: str = "float"              # "float" or "int"
     fallback: Optional[str] = None   # tensor to alias when this one is absent (tied head)
     # what the random-weights mode fills it with: "normal" (N(0, std)), "ones" (a gain: 1, or 1 + N(0, std)
     # with noisy gains) or "zeros"
     init: str = "normal"
+    # for "int" tensors in the random-weights mode: every row holds distinct values below ``high`` (0: zeros)
+    high: int = 0
 
 
 def canonical_name(name: str) -> str:
@@ -65,7 +67,7 @@ def storage_dtype(file_dtype: torch.dtype, kind: str, engine_dtype: torch.dtype)
 
 
 def check_names(expected: Mapping[str, WeightSpec],
-                found: Mapping[str, Tuple[int, ...]]) -> None:
+                found: Mapping[str, Tuple[int, ...]], ignorable=()) -> None:
     """Compare expected tensors with (canonical name -> shape) found; raise one WeightError."""
     exp = {canonical_name(n): (n, s) for n, s in expected.items()}
     missing: List[str] = []
@@ -76,9 +78,10 @@ def check_names(expected: Mapping[str, WeightSpec],
             if fb is None or fb not in found:
                 missing.append(n)
             continue
-        if tuple(found[cn]) != tuple(spec.shape):
+        if len(found[cn]) != len(spec.shape) or any(a != b and b != -1 for a, b in zip(found[cn], spec.shape)):
             wrong.append(f"{n}: expected {list(spec.shape)}, file has {list(found[cn])}")
-    unexpected = sorted(n for n in found if n not in exp)
+    skip = {canonical_name(n) for n in ignorable}
+    unexpected = sorted(n for n in found if n not in exp and n not in skip)
     if missing or wrong or unexpected:
         parts = []
         if missing:
@@ -92,7 +95,7 @@ def check_names(expected: Mapping[str, WeightSpec],
 
 
 def load_weights(folder: str, expected: Mapping[str, WeightSpec], engine_dtype: torch.dtype,
-                 device: torch.device | str) -> Dict[str, torch.Tensor]:
+                 device: torch.device | str, ignorable=()) -> Dict[str, torch.Tensor]:
     """Open every ``*.safetensors`` in ``folder``, check it against ``expected`` and
     return ``{expected name: tensor on device}``."""
     st = SafetensorsFolder(folder)
@@ -100,7 +103,7 @@ def load_weights(folder: str, expected: Mapping[str, WeightSpec], engine_dtype: 
         by_canon: Dict[str, str] = {}
         for n in st.names():
             by_canon[canonical_name(n)] = n
-        check_names(expected, {cn: st.entry(n).shape for cn, n in by_canon.items()})
+        check_names(expected, {cn: st.entry(n).shape for cn, n in by_canon.items()}, ignorable)
         out: Dict[str, torch.Tensor] = {}
         for name, spec in expected.items():
             cn = canonical_name(name)

@@ -36,10 +36,19 @@ def random_weights(expected: Mapping[str, WeightSpec], seed: int, dtype: torch.d
     for name, spec in expected.items():
         if spec.fallback is not None and tied:
             continue
+        if any(n < 0 for n in spec.shape):
+            raise ValueError(f"tensor '{name}': an axis of its shape {list(spec.shape)} is left to the checkpoint; "
+                             "random weights need every size")
         g = torch.Generator(device=device)
         g.manual_seed(_tensor_seed(seed, name))
         if spec.kind == "int":
-            out[name] = torch.zeros(spec.shape, dtype=torch.int32, device=device)
+            if spec.high > 0:       # every row: distinct values below ``high``, drawn without replacement
+                if len(spec.shape) != 2 or spec.shape[1] > spec.high:
+                    raise ValueError(f"tensor '{name}': rows of {spec.shape[1:]} distinct values below {spec.high}")
+                keys = torch.rand((spec.shape[0], spec.high), generator=g, dtype=torch.float32, device=device)
+                out[name] = keys.argsort(dim=1)[:, :spec.shape[1]].to(torch.int32).contiguous()
+            else:
+                out[name] = torch.zeros(spec.shape, dtype=torch.int32, device=device)
             continue
         if spec.init == "ones":
             t = torch.ones(spec.shape, dtype=torch.float32, device=device)
