@@ -428,11 +428,39 @@ def tosisun_shape(size, layers, vocab):
     return dict(architecture="Tosisun", width=z["width"], vocab=vocab, norm=dict(eps=1e-5), logit_softcap=30.0, layers=out)
 
 
+def tilivik_shape(size, layers, vocab):
+    """Layer sizes that resemble a real model's, for the Tilivik design: two layers of windowed softmax attention
+    (heads of 128 on the key/value heads of the Qwen2 model beside it, a window of 1,024 keys and 4 kept first
+    positions, capped scores, a bias by distance) beside gated linear attention (key channels of 64, values of 128),
+    then one of linear attention with a fixed decay per head; every feed-forward is a mixture of experts named by a
+    table; a run of two layers repeats, so that ``layers`` layers run (``layers`` - 2 hold tensors)."""
+    z = DESIGN_SIZES[size]
+    held = max(3, layers - 2)
+    out = []
+    for i in range(held):
+        mlp = dict(kind="moe", expert=dict(ff=z["expert_ff"]), router=dict(experts=z["experts"], top=z["top"]))
+        if i % 3 == 2:
+            nh = z["heads"]
+            mixer = dict(heads=nh, dim=128, vdim=128, decay=[1.0 - 2.0 ** (-2.0 - 6.0 * h / max(1, nh - 1)) for h in range(nh)])
+            out.append(dict(type="lightning", mixer=mixer, mlp=mlp))
+            continue
+        left = dict(heads=z["heads"], kv_heads=max(2, z["heads"] // 7), dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0,
+                    bias_max=4096, bias_rows=32, mask=dict(size=1024, keep_first=4))
+        right = dict(heads=z["heads"] // 2, dim=64, vdim=128, tau=16.0, rank=16)
+        out.append(dict(type="parallel", mlp=mlp, mixer=dict(left=left, right=right, left_scale=0.7, right_scale=0.7)))
+    cfg = dict(architecture="Tilivik", width=z["width"], vocab=vocab, norm=dict(eps=1e-6),
+               embedding=dict(bigram=dict(buckets=65521, mul_prev=31, mul_cur=17)), layers=out)
+    if layers > held:
+        cfg["loop"] = dict(start=1, stop=3, times=1 + (layers - held) // 2)
+    return cfg
+
+
 def design_comparison(args):
     """Prefill and decode of a model of the design at a real model's layer sizes, and of the benchmark's own
-    architecture (Qwen2 dense) at the same width, layers, heads and dense feed-forward, one after the other."""
+    architecture (Qwen2 dense) at the same width, layers, heads and dense feed-forward, one after the other; for
+    Tilivik also of Dedelorn, the nearest design the engine has (recurrent layers, a windowed attention, experts)."""
     import torch
-    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig, TosisunConfig
+    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig, TilivikConfig, TosisunConfig
     from zedinfer_amd.engine import Engine
     layers = args.layers if args.layers != FULL_LAYERS else 8
     vocab, prompt = 32000, args.prompt_len
@@ -441,7 +469,8 @@ def design_comparison(args):
     for size in (args.design_sizes.split(",") if args.design_sizes else ["1.5B"]):
         z = DESIGN_SIZES[size]
         design = {"dedelorn": lambda: (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn"),
-                  "tosisun": lambda: (TosisunConfig.from_dict(tosisun_shape(size, layers, vocab)), "Tosisun")}[args.design]
+                  "tosisun": lambda: (TosisunConfig.from_dict(tosisun_shape(size, layers, vocab)), "Tosisun"),
+                  "tilivik": lambda: (TilivikConfig.from_dict(tilivik_shape(size, layers, vocab)), "Tilivik")}[args.design]
         models = {
             args.design: design(),
             "qwen2": (Qwen2Config.from_dict(dict(SHAPE, hidden_size=z["width"], intermediate_size=z["ff"], vocab_size=vocab,
@@ -449,6 +478,10 @@ def design_comparison(args):
                                                  num_key_value_heads=max(2, z["heads"] // 7), tie_word_embeddings=False)),
                       "Qwen2ForCausalLM"),
         }
+        if args.design == "tilivik":
+            models["dedelorn"] = (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn")
+        if args.design_only:
+            models = {args.design: models[args.design]}
         rec = {}
         for name, (cfg, arch) in models.items():
             cache = {}
@@ -502,11 +535,12 @@ def main():
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     ap.add_argument("--resident-layer", action="store_true",
                     help="instead: time the one-launch decoder layer (ops.decode_layer) alone, --layers launches a step")
-    ap.add_argument("--design", default="", choices=["", "dedelorn", "tosisun"],
+    ap.add_argument("--design", default="", choices=["", "dedelorn", "tosisun", "tilivik"],
                     help="instead: prefill and decode of a model of this design at a real model's layer sizes, beside "
                          "Qwen2 dense of equal sizes (8 layers unless --layers says otherwise)")
     ap.add_argument("--design-sizes", default="", help="with --design: layer sizes, of " + ", ".join(sorted(DESIGN_SIZES)) +
                     " (commas between them; default 1.5B)")
+    ap.add_argument("--design-only", action="store_true", help="with --design: the design alone, no model beside it")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

@@ -108,6 +108,8 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
     half = rows // 2
     if n < half:
         return n
+    if half < 1 or far <= half:
+        return rows - 1
     return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
 
 
@@ -116,25 +118,32 @@ def visible(i: int, j: int, size: int, keep_first: int) -> bool:
 
 
 def biased_window_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m, eps: float) -> torch.Tensor:
+    """Dense over the whole sequence: a [T, T] matrix of scores per head, the bias and the visibility written out
+    pair by pair.  ``softcap``, ``bias_max`` (with the tensor ``rel``) and ``mask`` may each be absent."""
     H, G, dim, vdim = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
     T = h.shape[0]
     q = (h @ w["q"].T).view(T, H, dim)
     k = (h @ w["k"].T).view(T, G, dim)
     v = rms((h @ w["v"].T).view(T, G, vdim), eps)
-    rel = w["rel"]
-    rows = rel.shape[0]
-    cap, scale = float(m["softcap"]), float(m["scale"])
-    size, keep = int(m["mask"]["size"]), int(m["mask"]["keep_first"])
+    cap, scale = m.get("softcap"), float(m["scale"])
+    mask = m.get("mask")
+    size, keep = (int(mask["size"]), int(mask.get("keep_first", 0))) if mask else (T + 1, 0)
+    seen = torch.tensor([[visible(i, j, size, keep) for j in range(T)] for i in range(T)])
+    bucket = None
+    if m.get("bias_max") is not None:
+        rows = w["rel"].shape[0]
+        bucket = torch.tensor([[distance_bucket(i - j, rows, float(m["bias_max"])) if j <= i else 0 for j in range(T)]
+                               for i in range(T)])
     out = torch.zeros((T, H, vdim), dtype=F)
     for a in range(H):
         g = a // (H // G)
-        for i in range(T):
-            js = [j for j in range(i + 1) if visible(i, j, size, keep)]
-            s = torch.stack([q[i, a] @ k[j, g] for j in js]) * scale
-            s = cap * torch.tanh(s / cap)
-            s = s + torch.stack([rel[distance_bucket(i - j, rows, float(m["bias_max"])), a] for j in js])
-            p = torch.softmax(s, dim=0)
-            out[i, a] = (p[:, None] * v[js, g]).sum(dim=0)
+        s = (q[:, a] @ k[:, g].T) * scale
+        if cap:
+            s = float(cap) * torch.tanh(s / float(cap))
+        if bucket is not None:
+            s = s + w["rel"][:, a][bucket]
+        s = s.masked_fill(~seen, float("-inf"))
+        out[:, a] = torch.softmax(s, dim=1) @ v[:, g]
     y = out.reshape(T, H * vdim) * torch.sigmoid(h @ w["g"].T)
     return y @ w["o"].T
 
@@ -230,3 +239,12 @@ class PlainTilivik:
             if streams is not None:
                 streams.append(x.clone())
         return scalar_norm(x, self.t["final.norm"], self.eps) @ self.t["head"].T
+
+    def greedy_generate(self, prompt: Sequence[int], new_tokens: int) -> List[int]:
+        """The tokens greedy decoding appends (the lowest index among equal logits), each from a full forward pass."""
+        toks, out = list(prompt), []
+        for _ in range(new_tokens):
+            nxt = int(torch.argmax(self.forward(toks)[-1]))
+            out.append(nxt)
+            toks.append(nxt)
+        return out
