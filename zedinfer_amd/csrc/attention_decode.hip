@@ -68,7 +68,15 @@ struct DecProjection {
     int write_kv;
 };
 
-template <int D, bool FUSED, int VMODE>
+// exp2-based tanh: 1 - 2 / (2^(2 x log2 e) + 1), right at both ends
+__device__ __forceinline__ float dec_tanh(float x) {
+    return 1.f - 2.f / (__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
+}
+
+// BIASED: the scores are capped and biased by distance, and the sequence's first positions stay visible beside the
+// window (ZiScoreExtras); those of them that lie below the token's window are walked by the first wavefront of the
+// token's first chunk, before its own keys.
+template <int D, bool FUSED, int VMODE, bool BIASED>
 __global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE, 2)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
@@ -76,8 +84,10 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                         int max_pages, int num_pages, int nh, int nkv, int G, int ps, int window, float scale,
-                        int max_chunks, int leave_parts, DecProjection pj, const float* __restrict__ sinks) {
+                        int max_chunks, int leave_parts, DecProjection pj, const float* __restrict__ sinks,
+                        ZiScoreExtras ex) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
+    static_assert(!(FUSED && BIASED), "the kernel that rotates and stores has plain scores");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DT = D / 16;          // output tiles of 16 dims
     constexpr bool WHOLE_LINES = D % 64 == 0;   // a key is whole 128-byte lines: see the loads of the keys
@@ -274,7 +284,11 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     float m = -INFINITY, lsum = 0.f;   // m is in base-2 units: the maximum of s * scale * log2(e)
     const float scale_log2 = scale * 1.4426950408889634f;
 
-    for (int base = k_begin; base < k_end; base += DEC_BLOCK) {
+    // the kept first positions below the window: [0, kept_end), for one wavefront of the token
+    const int kept_end = (BIASED && chunk == 0 && wave == 0) ? (ex.keep_first < sp.lo ? ex.keep_first : sp.lo) : 0;
+    for (int phase = kept_end > 0 ? 0 : 1; phase < 2; ++phase) {
+    const int key_lo = phase ? sp.lo : 0, key_end = phase ? k_end : kept_end;      // the keys that count: [key_lo, key_end)
+    for (int base = phase ? k_begin : 0; base < key_end; base += DEC_BLOCK) {
         // ---- all loads of the block first, in straight-line code: the six table lookups, then keys
         // (4 tiles x DK) and values (DT x 2) from addresses clamped into the sequence and the pool.  What
         // must not count is masked afterwards; with a branch around a load the compiler would wait for it
@@ -398,7 +412,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         }
         // Keys outside [lo, p] get the score -inf below, whatever was loaded for them.  Their values
         // must be zero, since 0 * NaN is NaN: slots outside the range may hold anything.
-        if (base < sp.lo || base + DEC_BLOCK > k_end) {
+        if (base < key_lo || base + DEC_BLOCK > key_end) {
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 const int key0 = zi_dec_value_key0(base, b, j);
@@ -406,7 +420,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int ka = key0 + 2 * e, kb2 = ka + 1;
-                    keep[e] = ((ka >= sp.lo && ka < k_end) ? 0xffffu : 0u) | ((kb2 >= sp.lo && kb2 < k_end) ? 0xffff0000u : 0u);
+                    keep[e] = ((ka >= key_lo && ka < key_end) ? 0xffffu : 0u) | ((kb2 >= key_lo && kb2 < key_end) ? 0xffff0000u : 0u);
                 }
 #pragma unroll
                 for (int dd = 0; dd < DT; ++dd) {
@@ -450,14 +464,29 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                 s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[tt][dk].b, qop[dk], s[tt], 0, 0, 0);
         }
         // softmax in base 2: t = s * scale * log2(e), p = 2^(t - m)
-        const bool whole = base >= sp.lo && base + DEC_BLOCK <= k_end;
+        const bool whole = base >= key_lo && base + DEC_BLOCK <= key_end;
         float mx = -INFINITY;
+        const float inv_cap = (BIASED && ex.softcap > 0.f) ? 1.f / ex.softcap : 0.f;
+        const float* brow = (BIASED && ex.bias) ? ex.bias + (int64_t)(kvh * G + (r < G ? r : G - 1)) * ex.bias_len : nullptr;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int key = zi_dec_score_key(base, tt, j, e);
-                const float v = (whole || (key >= sp.lo && key < k_end)) ? s[tt][e] * scale_log2 : -INFINITY;
+                float sc;
+                if constexpr (BIASED) {
+                    sc = s[tt][e] * scale;
+                    if (ex.softcap > 0.f) sc = ex.softcap * dec_tanh(sc * inv_cap);
+                    if (brow) {
+                        int dist = p - key;
+                        dist = dist < 0 ? 0 : (dist < ex.bias_len ? dist : ex.bias_len - 1);
+                        sc += brow[dist];
+                    }
+                    sc *= 1.4426950408889634f;
+                } else {
+                    sc = s[tt][e] * scale_log2;
+                }
+                const float v = (whole || (key >= key_lo && key < key_end)) ? sc : -INFINITY;
                 s[tt][e] = v;
                 mx = fmaxf(mx, v);
             }
@@ -491,6 +520,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
             for (int b = 0; b < 2; ++b)
                 o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dd][b].b, pb[b].b, o[dd], 0, 0, 0);
         }
+    }
     }
     // ---- merge the four wavefronts: head r's (m, l) and this lane's outputs
     lsum += __shfl_xor(lsum, 16, ZI_WAVE);
@@ -737,7 +767,11 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
                       const void* kcache, const void* vcache, const int32_t* tok_index, const int32_t* tok_seq,
                       const int32_t* tok_pos, const int32_t* block_tables, int max_pages, int num_pages, int nh, int nkv,
                       int d, int page_size, int window, float scale, int max_chunks, float* workspace,
-                      int64_t workspace_floats, const DecProjection* pj, const float* sinks, hipStream_t stream) {
+                      int64_t workspace_floats, const DecProjection* pj, const float* sinks, hipStream_t stream,
+                      ZiScoreExtras ex = ZiScoreExtras{0.f, nullptr, 0, 0}) {
+    const bool biased = ex.softcap > 0.f || ex.bias != nullptr || ex.keep_first > 0;
+    ZI_REQUIRE(!(biased && pj), "%s: capped or biased scores come with queries that are made beforehand", who);
+    ZI_REQUIRE(ex.softcap >= 0.f && ex.keep_first >= 0 && (!ex.bias || ex.bias_len > 0), "%s: bad cap, bias or kept positions", who);
     ZI_REQUIRE(zi_attention_decode_supported(dt, nh, nkv, d, page_size),
                "%s: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, group <= 16, "
                "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", who, dt, nh, nkv, d, page_size);
@@ -763,15 +797,20 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
     const DecProjection none = {};
 #define ZI_DEC(DD, VMODE)                                                                                            \
     if (pj)                                                                                                          \
-        attention_decode_kernel<DD, true, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+        attention_decode_kernel<DD, true, VMODE, false><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                   \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, leave_parts, *pj, sinks);                                                                                      \
+            max_chunks, leave_parts, *pj, sinks, ex);                                                                \
+    else if (biased)                                                                                                 \
+        attention_decode_kernel<DD, false, VMODE, true><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                   \
+            (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
+            tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
+            max_chunks, leave_parts, none, sinks, ex);                                                               \
     else                                                                                                             \
-        attention_decode_kernel<DD, false, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
+        attention_decode_kernel<DD, false, VMODE, false><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                  \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, leave_parts, none, sinks)
+            max_chunks, leave_parts, none, sinks, ex)
     switch (d) {
         case 16: ZI_DEC(16, 0); break;
         case 32: ZI_DEC(32, 0); break;
@@ -817,6 +856,21 @@ extern "C" int zi_attention_decode_sink(void* out, const void* q, int dt, int n_
     return dec_launch("attention_decode_sink", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
                       block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
                       workspace_floats, nullptr, sinks, stream);
+}
+
+// The same with capped and biased scores and kept first positions (ZiScoreExtras): `softcap` 0 for none, `bias`
+// float32 [nh][bias_len] or null, `keep_first` positions of every sequence stay visible beside the window.
+extern "C" int zi_attention_decode_biased(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
+                                          const void* kcache, const void* vcache, const int32_t* tok_index,
+                                          const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                          int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                                          float scale, int max_chunks, float* workspace, int64_t workspace_floats,
+                                          const float* sinks, float softcap, const float* bias, int bias_len,
+                                          int keep_first, hipStream_t stream) {
+    ZI_REQUIRE(out != nullptr, "attention_decode_biased: the chunks are merged here");
+    return dec_launch("attention_decode_biased", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
+                      block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
+                      workspace_floats, nullptr, sinks, stream, ZiScoreExtras{softcap, bias, bias_len, keep_first});
 }
 
 // 1 when the fused entry point takes this projection layout, else 0 (then: rotate and store first, and

@@ -61,7 +61,15 @@ __device__ __forceinline__ uint4 pf_keep(uint4 v, int keep) {
     return make_uint4(v.x & mask, v.y & mask, v.z & mask, v.w & mask);
 }
 
-template <int D>
+// exp2-based tanh: 1 - 2 / (2^(2 x log2 e) + 1), right at both ends (2^inf = inf gives 1, 2^-inf = 0 gives -1)
+__device__ __forceinline__ float pf_tanh(float x) {
+    return 1.f - 2.f / (__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
+}
+
+// BIASED: the scores are capped and biased by distance, and the sequence's first positions stay visible beside the
+// window (ZiScoreExtras).  The blocks of those first positions that lie below the tile's walk are walked first, by
+// the workgroup of the tile's first cut.
+template <int D, bool BIASED>
 __global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
 attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
                          const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
@@ -70,7 +78,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                          const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
                          int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
                          float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int chunk_keys,
-                         const float* __restrict__ sinks) {
+                         const float* __restrict__ sinks, ZiScoreExtras ex) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
@@ -236,7 +244,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         const int kb = kb0 + kh * PF_BN;      // this wavefront's 64 keys of the block
         const uint16_t* kl = k_lds + cur * (PF_BS * KS) + kh * (PF_BN * KS);
         const uint16_t* vl = v_lds + cur * (D * VS) + kh * PF_BN;
-        if (wave_active && kb <= wave_last && kb + PF_BN > wave_lo) {
+        if (wave_active && kb <= wave_last && (kb + PF_BN > wave_lo || (BIASED && kb < ex.keep_first))) {
         // ---- scores of 64 keys for this lane's query
         pf_f32x4_t s[4];
 #pragma unroll
@@ -251,9 +259,30 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         }
         // softmax in base 2: t = s * scale * log2(e), p = 2^(t - m).  A block that every query of the
         // wavefront sees whole (all but those on the diagonal and at a window's edge) needs no mask.
-        const bool whole = kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
+        const bool whole = !BIASED && kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
         float mx = -INFINITY;
-        if (whole) {
+        if constexpr (BIASED) {
+            // every score becomes its capped and biased value, in base-2 units already
+            const float inv_cap = ex.softcap > 0.f ? 1.f / ex.softcap : 0.f;
+            const float* brow = ex.bias ? ex.bias + (int64_t)h * ex.bias_len : nullptr;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                    const bool vis = key <= qpos && (window <= 0 || key > qpos - window || key < ex.keep_first);
+                    float sc = s[t][x] * scale;
+                    if (ex.softcap > 0.f) sc = ex.softcap * pf_tanh(sc * inv_cap);
+                    if (brow) {
+                        int dist = qpos - key;
+                        dist = dist < 0 ? 0 : (dist < ex.bias_len ? dist : ex.bias_len - 1);
+                        sc += brow[dist];
+                    }
+                    const float v = vis ? sc * 1.4426950408889634f : -INFINITY;
+                    s[t][x] = v;
+                    mx = fmaxf(mx, v);
+                }
+        } else if (whole) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -274,7 +303,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
         // the scale is positive (the host checks): the largest scaled score is the largest score, scaled; the
         // scaling of every score is then one fused multiply-add with the subtraction of the maximum
-        const float m_new = fmaxf(m, mx * scale_log2);
+        const float to_log2 = BIASED ? 1.f : scale_log2;
+        const float m_new = fmaxf(m, mx * to_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float corr = __builtin_amdgcn_exp2f(m - m_use);      // 2^(-inf) = 0 before the first key
         m = m_new;
@@ -283,7 +313,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                s[t][x] = __builtin_amdgcn_exp2f(fmaf(s[t][x], scale_log2, -m_use));    // 0 for masked keys
+                s[t][x] = __builtin_amdgcn_exp2f(fmaf(s[t][x], to_log2, -m_use));    // 0 for masked keys
                 psum += s[t][x];
             }
         pf_pack pb[2];
@@ -312,6 +342,20 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
             }
         }
     };
+    if constexpr (BIASED) {
+        // the blocks of the kept first positions that lie below this tile's walk (its first cut walks them),
+        // through the second LDS buffer: the first already holds the walk's first block
+        if (window > 0 && blockIdx.y == 0) {
+            const int kept_end = ex.keep_first < kb_begin ? ex.keep_first : kb_begin;
+            for (int kbx = 0; kbx < kept_end; kbx += PF_BS) {
+                fetch(kbx);
+                stash(kbx, 1);
+                __syncthreads();
+                work(kbx, 1);
+                __syncthreads();
+            }
+        }
+    }
     // The next block travels from the cache into registers while this one is worked on; it goes into
     // the other LDS buffer, which everyone has finished reading at the barrier before.  The last block
     // stands outside the loop, so that no branch surrounds the loop's loads.
@@ -850,13 +894,20 @@ extern "C" int zi_attention_prefill_cuts(int max_keys, int window, int groups, i
 // tiles; a query's keys are then added in another order, so the result differs by rounding.
 // `sinks` (float32 [nh], or null): the softmax of head h also counts exp(sinks[h]) in its denominator, once, whatever
 // the number of cuts of a tile's keys.
-extern "C" int zi_attention_prefill_sink(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
-                                         const void* kcache, const void* vcache, const int32_t* tile_entry,
-                                         const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
-                                         const int32_t* entry_past, const int32_t* block_tables, int max_pages,
-                                         int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
-                                         int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
-                                         int alone, int chunk_keys, const float* sinks, hipStream_t stream) {
+// `softcap`, `bias` (float32 [nh][bias_len]) and `keep_first`: see ZiScoreExtras; with any of them tiles hold 64
+// queries and the kernel that stages through registers runs for every head size.
+extern "C" int zi_attention_prefill_biased(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
+                                           const void* kcache, const void* vcache, const int32_t* tile_entry,
+                                           const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
+                                           const int32_t* entry_past, const int32_t* block_tables, int max_pages,
+                                           int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                           int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
+                                           int alone, int chunk_keys, const float* sinks, float softcap,
+                                           const float* bias, int bias_len, int keep_first, hipStream_t stream) {
+    const bool biased = softcap > 0.f || bias != nullptr || keep_first > 0;
+    ZI_REQUIRE(softcap >= 0.f && keep_first >= 0 && (!bias || bias_len > 0), "attention_prefill: bad cap, bias or kept positions");
+    ZI_REQUIRE(!biased || (tile == PF_BM && !alone), "attention_prefill: capped or biased scores and kept positions take tiles of %d queries", PF_BM);
+    const ZiScoreExtras ex = {softcap, bias, bias_len, keep_first};
     ZI_REQUIRE(tile == PF_BM || (tile == 2 * PF_BM && pf_variant >= 1 && (d == 64 || d == 128)),
                "attention_prefill: tiles of %d queries (64, or 128 for head sizes 64 and 128)", tile);
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
@@ -885,16 +936,22 @@ extern "C" int zi_attention_prefill_sink(void* out, const void* q, int dt, int n
     float* po = workspace;
     float* pml = workspace ? workspace + (int64_t)rows * nh * max_chunks * d : nullptr;
 #define ZI_PF(DD)                                                                                              \
-    attention_prefill_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                     \
-        (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
-        tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
-        window, scale, po, pml, max_chunks, chunk_keys, sinks)
+    if (biased)                                                                                                \
+        attention_prefill_kernel<DD, true><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                           \
+            (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
+            tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift, \
+            window, scale, po, pml, max_chunks, chunk_keys, sinks, ex);                                        \
+    else                                                                                                       \
+        attention_prefill_kernel<DD, false><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                          \
+            (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
+            tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift, \
+            window, scale, po, pml, max_chunks, chunk_keys, sinks, ex)
 #define ZI_PF_DMA(DD, QW, KH)                                                                                  \
     attention_prefill_dma_kernel<DD, QW, KH><<<grid, 4 * KH * ZI_WAVE, 0, stream>>>(                           \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks, chunk_keys, sinks)
-    const bool dma = pf_variant >= 1 && (d == 64 || d == 128);
+    const bool dma = !biased && pf_variant >= 1 && (d == 64 || d == 128);
     const bool wide = tile == 2 * PF_BM;
     ZI_REQUIRE(!alone || dma, "attention_prefill: workgroups of four wavefronts are for head sizes 64 and 128");
     if (dma && d == 128 && wide && alone) ZI_PF_DMA(128, 2, 1);
@@ -923,6 +980,19 @@ extern "C" int zi_attention_prefill_sink(void* out, const void* q, int dt, int n
             (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks,
             tile, chunk_keys, sinks);
     return zi_check_launch("attention_prefill");
+}
+
+extern "C" int zi_attention_prefill_sink(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
+                                         const void* kcache, const void* vcache, const int32_t* tile_entry,
+                                         const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
+                                         const int32_t* entry_past, const int32_t* block_tables, int max_pages,
+                                         int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                         int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
+                                         int alone, int chunk_keys, const float* sinks, hipStream_t stream) {
+    return zi_attention_prefill_biased(out, q, dt, num_tiles, ldq, ldo, kcache, vcache, tile_entry, tile_off, entry_start,
+                                       entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, d, page_size,
+                                       window, scale, rows, max_chunks, workspace, workspace_floats, tile, alone,
+                                       chunk_keys, sinks, 0.f, nullptr, 0, 0, stream);
 }
 
 extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,

@@ -17,7 +17,9 @@
 #include "zi_api.h"
 
 #define LA_COLS 4                       // columns of S a wavefront holds
-#define LA_PARTS (ZI_WAVE / LA_COLS)    // lanes that share a column: lane (c, p) holds rows p, p + 16, ...
+#define LA_PARTS (ZI_WAVE / LA_COLS)    // lanes that share a column: lane (c, p) holds rows p * R .. p * R + R - 1
+#define LA_WAVES 4                      // wavefronts of a workgroup: they share the staged tokens
+#define LA_WCOLS (LA_COLS * LA_WAVES)   // columns of S a workgroup holds
 
 __device__ __forceinline__ float la_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float la_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
@@ -53,77 +55,162 @@ extern "C" int zi_lowrank_decay(float* out, int64_t ldo, const float* u, int64_t
     return zi_check_launch("lowrank_decay");
 }
 
-// One wavefront per (entry, head, LA_COLS columns of S).  R rows a lane.  The next token's operands are asked
-// for before the present token is worked on.
-template <int R>
-__global__ void __launch_bounds__(ZI_WAVE)
+// x of the lane that `CTRL` names within this lane's row of 16 lanes (quad permutations, mirrors)
+template <int CTRL>
+__device__ __forceinline__ float la_dpp(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+// the sum over the 16 lanes of a row, in every one of them
+__device__ __forceinline__ float la_row_sum(float x) {
+    x += la_dpp<0xB1>(x);       // quad_perm [1, 0, 3, 2]
+    x += la_dpp<0x4E>(x);       // quad_perm [2, 3, 0, 1]
+    x += la_dpp<0x141>(x);      // row_half_mirror
+    x += la_dpp<0x140>(x);      // row_mirror
+    return x;
+}
+
+// where element e of a staged row lies: 16 bytes are skipped every 64 floats, so that the 16-byte reads of the
+// sixteen lanes of a row (lane p reads R consecutive floats from p * R) fall into different banks
+__device__ __forceinline__ constexpr int la_place(int e) { return e + (e >> 6) * 4; }
+
+// A workgroup of LA_WAVES wavefronts per (entry, head, LA_WCOLS columns of S); a wavefront holds LA_COLS of
+// them, lane (c, p) rows p * R .. p * R + R - 1 of column c in registers.  k, q (and the decays) of TC tokens at a
+// time lie in LDS, activated and scaled as they are put there (once, not by every lane that reads them); the next
+// TC tokens are asked for before the present ones are worked on and go into the other buffer afterwards, so no
+// token waits for memory.  Nothing but the state's own multiply-add chains one token to the next: the read-outs
+// of a chunk's tokens are summed over the lanes together, after the chunk.
+template <int R, int TC, bool GATED>
+__global__ void __launch_bounds__(LA_WAVES* ZI_WAVE)
 linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ q, const float* __restrict__ k,
                         const float* __restrict__ v, int64_t ld, const float* __restrict__ decay, int64_t ld_decay,
                         const float* __restrict__ head_decay, float* __restrict__ state, int64_t state_stride,
                         const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                         const int32_t* __restrict__ entry_past, const int32_t* __restrict__ entry_slot, int heads,
                         int dim, int vdim, int act, float qscale) {
-    const int lane = threadIdx.x, c = lane / LA_PARTS, p = lane % LA_PARTS;
+    constexpr int D = LA_PARTS * R;               // rows the lanes of a column hold
+    constexpr int DP = la_place(D);               // floats of a staged row
+    constexpr int NSEG = GATED ? 3 : 2;           // k, q (, decay)
+    constexpr int THREADS = LA_WAVES * ZI_WAVE;
+    constexpr int NE = TC * NSEG * D;
+    constexpr int PRE = (NE + THREADS - 1) / THREADS;
+    static_assert(TC <= LA_PARTS && TC * LA_WCOLS <= THREADS, "a chunk's read-outs are written by the lanes of a row");
+    __shared__ __attribute__((aligned(16))) float rows[2][TC][NSEG][DP];
+    __shared__ float vs[2][TC][LA_WCOLS];
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int c = lane / LA_PARTS, p = lane % LA_PARTS;
     const int head = blockIdx.y, e = blockIdx.z;
-    const int col = blockIdx.x * LA_COLS + c;
+    const int col0 = blockIdx.x * LA_WCOLS, col = col0 + wave * LA_COLS + c;
     const bool live = col < vdim;
     const int colc = live ? col : vdim - 1;
     const int t0 = entry_start[e], len = entry_len[e];
+    if (len <= 0) return;
     float* S_ = state + (int64_t)entry_slot[e] * state_stride + (int64_t)head * dim * vdim;
     const bool fresh = entry_past[e] == 0;      // a sequence's first tokens: the state is zero whatever the slot holds
     float S[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int row = r * LA_PARTS + p;
+        const int row = p * R + r;
         S[r] = (!fresh && row < dim) ? S_[(int64_t)row * vdim + colc] : 0.f;
     }
     const float hd = head_decay ? head_decay[head] : 1.f;
-    const int64_t qk_at = (int64_t)head * dim, v_at = (int64_t)head * vdim + colc;
-    float kq[R], qq[R], aq[R], vq;
-    auto load = [&](int t, float* kk, float* qv, float* av, float& vv) {
-        const int64_t base = (int64_t)t * ld;
+    const int64_t qk_at = (int64_t)head * dim, v_at = (int64_t)head * vdim;
+
+    // global -> registers: the chunk of tokens from `base` on.  Every load is issued, from addresses clamped into
+    // the entry; what a thread must not use is zeroed when it goes to LDS.
+    float pre[PRE], vpre;
+    unsigned ok_bits = 0;
+    bool v_ok = false;
+    auto fetch = [&](int base) {
+        const int n_in = len - base;      // tokens of the chunk (more than TC: all TC; none or fewer past the end)
+        const int tb = t0 + (base < len ? base : len - 1);
+        ok_bits = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = r * LA_PARTS + p;
-            const bool in = row < dim;
-            kk[r] = in ? k[base + qk_at + row] : 0.f;
-            qv[r] = in ? q[base + qk_at + row] : 0.f;
-            av[r] = decay ? (in ? decay[(int64_t)t * ld_decay + qk_at + row] : 0.f) : hd;
+        for (int i = 0; i < PRE; ++i) {
+            const int idx = i * THREADS + tid;
+            const int tt = idx / (NSEG * D), rem = idx % (NSEG * D), seg = rem / D, d = rem % D;
+            const bool ok = idx < NE && tt < n_in && d < dim;
+            const int64_t tok = tb + (ok ? tt : 0);
+            const int dd = ok ? d : 0;
+            const float* src = seg == 0 ? k : (seg == 1 ? q : decay);
+            pre[i] = src[tok * (seg == 2 ? ld_decay : ld) + qk_at + dd];
+            ok_bits |= (unsigned)ok << i;
         }
-        vv = v[base + v_at];
+        const int tt = tid / LA_WCOLS, cc = tid % LA_WCOLS;
+        v_ok = tid < TC * LA_WCOLS && tt < n_in && col0 + cc < vdim;
+        vpre = v[(int64_t)(tb + (v_ok ? tt : 0)) * ld + v_at + (v_ok ? col0 + cc : 0)];
     };
-    if (len > 0) load(t0, kq, qq, aq, vq);
-    for (int i = 0; i < len; ++i) {
-        float kn[R], qn[R], an[R], vn = 0.f;
-        if (i + 1 < len) load(t0 + i + 1, kn, qn, an, vn);
-        float vv = vq;
-        if (act) vv = la_silu(vv);
-        float acc = 0.f;
+    auto stash = [&](int b) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            float kk = kq[r], qv = qq[r];
-            if (act) {
-                kk = la_silu(kk);
-                qv = la_silu(qv);
+        for (int i = 0; i < PRE; ++i) {
+            const int idx = i * THREADS + tid;
+            if (idx >= NE) continue;
+            const int tt = idx / (NSEG * D), rem = idx % (NSEG * D), seg = rem / D, d = rem % D;
+            float x = ((ok_bits >> i) & 1u) ? pre[i] : 0.f;
+            if (seg < 2 && act) x = la_silu(x);
+            if (seg == 1) x *= qscale;
+            rows[b][tt][seg][la_place(d)] = x;
+        }
+        if (tid < TC * LA_WCOLS) {
+            const float x = v_ok ? vpre : 0.f;
+            vs[b][tid / LA_WCOLS][tid % LA_WCOLS] = act ? la_silu(x) : x;
+        }
+    };
+    auto work = [&](int base, int b) {
+        const int n_in = len - base;
+        float accs[TC];
+#pragma unroll
+        for (int tt = 0; tt < TC; ++tt) {
+            accs[tt] = 0.f;
+            if (tt < n_in) {
+                float kk[R], qq[R], aa[R];
+                const float* kr = &rows[b][tt][0][la_place(p * R)];
+                const float* qr = &rows[b][tt][1][la_place(p * R)];
+                if constexpr (R == 2) {
+                    *reinterpret_cast<float2*>(kk) = *reinterpret_cast<const float2*>(kr);
+                    *reinterpret_cast<float2*>(qq) = *reinterpret_cast<const float2*>(qr);
+                    if constexpr (GATED) *reinterpret_cast<float2*>(aa) = *reinterpret_cast<const float2*>(&rows[b][tt][NSEG - 1][la_place(p * R)]);
+                } else {
+#pragma unroll
+                    for (int r4 = 0; r4 < R; r4 += 4) {
+                        *reinterpret_cast<float4*>(kk + r4) = *reinterpret_cast<const float4*>(kr + r4);
+                        *reinterpret_cast<float4*>(qq + r4) = *reinterpret_cast<const float4*>(qr + r4);
+                        if constexpr (GATED)
+                            *reinterpret_cast<float4*>(aa + r4) = *reinterpret_cast<const float4*>(&rows[b][tt][NSEG - 1][la_place(p * R)] + r4);
+                    }
+                }
+                const float vv = vs[b][tt][wave * LA_COLS + c];
+                float acc = 0.f;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    S[r] = (GATED ? aa[r] : hd) * S[r] + kk[r] * vv;
+                    acc += S[r] * qq[r];
+                }
+                accs[tt] = acc;
             }
-            S[r] = aq[r] * S[r] + kk * vv;
-            acc += S[r] * (qv * qscale);
         }
+        float mine = 0.f;
 #pragma unroll
-        for (int o = LA_PARTS / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, ZI_WAVE);
-        if (p == 0 && live) out[(int64_t)(t0 + i) * ldo + (int64_t)head * vdim + col] = acc;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            kq[r] = kn[r];
-            qq[r] = qn[r];
-            aq[r] = an[r];
+        for (int tt = 0; tt < TC; ++tt) {
+            const float total = la_row_sum(accs[tt]);
+            if (p == tt) mine = total;
         }
-        vq = vn;
+        // lane (c, p) writes token p's read-out of column c
+        if (live && p < TC && p < n_in) out[(int64_t)(t0 + base + p) * ldo + (int64_t)head * vdim + col] = mine;
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int cur = 0;
+    for (int base = 0; base < len; base += TC, cur ^= 1) {
+        fetch(base + TC);
+        work(base, cur);
+        stash(cur ^ 1);
+        __syncthreads();
     }
-    if (live && len > 0) {
+    if (live) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = r * LA_PARTS + p;
+            const int row = p * R + r;
             if (row < dim) S_[(int64_t)row * vdim + col] = S[r];
         }
     }
@@ -146,16 +233,21 @@ extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, cons
                (!decay || ld_decay >= (int64_t)heads * dim), "linear_attention: row stride too small");
     ZI_REQUIRE(act == 0 || act == 1, "linear_attention: unknown activation %d", act);
     if (entries == 0) return 0;
-    const dim3 grid((vdim + LA_COLS - 1) / LA_COLS, heads, entries);
-#define ZI_LA(R)                                                                                                    \
-    linear_attention_kernel<R><<<grid, ZI_WAVE, 0, stream>>>(out, ldo, q, k, v, ld, decay, ld_decay, head_decay,    \
-                                                             state, state_stride, entry_start, entry_len, entry_past, \
-                                                             entry_slot, heads, dim, vdim, act, qscale)
-    if (dim <= 32) ZI_LA(2);
-    else if (dim <= 64) ZI_LA(4);
-    else if (dim <= 128) ZI_LA(8);
-    else if (dim <= 256) ZI_LA(16);
-    else ZI_LA(32);
+    const dim3 grid((vdim + LA_WCOLS - 1) / LA_WCOLS, heads, entries);
+#define ZI_LA(R, TC)                                                                                                 \
+    if (decay)                                                                                                       \
+        linear_attention_kernel<R, TC, true><<<grid, LA_WAVES * ZI_WAVE, 0, stream>>>(                               \
+            out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride, entry_start, entry_len,         \
+            entry_past, entry_slot, heads, dim, vdim, act, qscale);                                                  \
+    else                                                                                                             \
+        linear_attention_kernel<R, TC, false><<<grid, LA_WAVES * ZI_WAVE, 0, stream>>>(                              \
+            out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride, entry_start, entry_len,         \
+            entry_past, entry_slot, heads, dim, vdim, act, qscale)
+    if (dim <= 32) { ZI_LA(2, 16); }
+    else if (dim <= 64) { ZI_LA(4, 16); }
+    else if (dim <= 128) { ZI_LA(8, 16); }
+    else if (dim <= 256) { ZI_LA(16, 8); }
+    else { ZI_LA(32, 4); }
 #undef ZI_LA
     return zi_check_launch("linear_attention");
 }

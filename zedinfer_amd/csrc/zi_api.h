@@ -233,6 +233,19 @@ int zi_attention_generic_biased(void* out, const void* q, int dt, int n, int64_t
     const void* vcache, const int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
     block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, const
     float* sinks, float softcap, const float* bias, int bias_len, int keep_first, hipStream_t stream);
+// attention_prefill.hip
+int zi_attention_prefill_biased(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo, const void*
+    kcache, const void* vcache, const int32_t* tile_entry, const int32_t* tile_off, const int32_t* entry_start, const
+    int32_t* entry_len, const int32_t* entry_past, const int32_t* block_tables, int max_pages, int num_pages, int nh,
+    int nkv, int d, int page_size, int window, float scale, int rows, int max_chunks, float* workspace, int64_t
+    workspace_floats, int tile, int alone, int chunk_keys, const float* sinks, float softcap, const float* bias, int
+    bias_len, int keep_first, hipStream_t stream);
+// attention_decode.hip
+int zi_attention_decode_biased(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo, const void* kcache,
+    const void* vcache, const int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, int
+    max_chunks, float* workspace, int64_t workspace_floats, const float* sinks, float softcap, const float* bias, int
+    bias_len, int keep_first, hipStream_t stream);
 // moe.hip
 int zi_moe_route_table(int32_t* idx, float* wt, const int32_t* ids, const int32_t* table, int n, int vocab, int
     experts, int top, hipStream_t stream);
@@ -303,6 +316,8 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_gated_rmsnorm_act) \
     X(zi_normed_kv_store) \
     X(zi_attention_generic_biased) \
+    X(zi_attention_prefill_biased) \
+    X(zi_attention_decode_biased) \
     X(zi_moe_route_table) \
     X(zi_argmax) \
     X(zi_sample)

@@ -21,6 +21,17 @@
 #define ZI_HD inline
 #endif
 
+// ---- what a softmax mixer may do to a score beside scaling it --------------------------------------
+// score = (q . k) * scale; then softcap * tanh(score / softcap) when softcap > 0; then + bias[head][min(distance,
+// bias_len - 1)] when bias is not null (float32 [heads][bias_len], distance = query position - key position); beside
+// the window, the sequence's first keep_first positions stay visible.
+struct ZiScoreExtras {
+    float softcap;
+    const float* bias;
+    int bias_len;
+    int keep_first;
+};
+
 // ---- places in the pool --------------------------------------------------------------------------
 ZI_HD int64_t zi_key_offset(int64_t page, int kv_head, int slot_in_page, int nkv, int ps, int d) {
     return ((page * nkv + kv_head) * ps + slot_in_page) * d;          // + dim

@@ -107,6 +107,9 @@ _PROTOTYPES = {
     "zi_gated_rmsnorm_act": [P, I, L, P, P, I, P, L, I, I, I, F, I, F, P],
     "zi_normed_kv_store": [P, I, L, P, P, P, L, I, I, I, P, L, I, I, I, I, I, I, I, F, I, P],
     "zi_attention_generic_biased": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, F, P, I, I, P],
+    "zi_attention_prefill_biased": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I,
+                                    P, F, P, I, I, P],
+    "zi_attention_decode_biased": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P, F, P, I, I, P],
     "zi_moe_route_table": [P, P, P, P, I, I, I, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
     "zi_tape_record_many": [P, c_char_p, P, P, I],

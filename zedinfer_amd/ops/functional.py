@@ -411,16 +411,36 @@ def attention_decode_workspace(tokens: int, nh: int, d: int) -> int:
     return int(_lib.load().zi_attention_decode_workspace(int(tokens), int(nh), int(d)))
 
 
+def _score_extras(who: str, nh: int, q: torch.Tensor, softcap: float, bias: Optional[torch.Tensor], keep_first: int):
+    """(softcap, bias pointer, distances of the bias, kept positions) for the entry points that take capped and
+    biased scores; None when none of them is asked for."""
+    if not (softcap and softcap > 0) and bias is None and not keep_first:
+        return None
+    L = 0
+    if bias is not None:
+        if bias.dtype != torch.float32 or bias.dim() != 2 or bias.shape[0] != nh or not bias.is_contiguous() \
+                or bias.device != q.device or bias.shape[1] < 1:
+            raise ValueError(f"{who}: the bias must be a contiguous float32 [{nh}, distances] tensor on {q.device}")
+        L = int(bias.shape[1])
+    if softcap < 0 or keep_first < 0:
+        raise ValueError(f"{who}: the cap and the kept positions cannot be negative")
+    return (float(softcap or 0.0), _p(bias), L, int(keep_first))
+
+
 def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
                      tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                      max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
                      tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                     sinks: Optional[torch.Tensor] = None, leave_chunks: bool = False) -> Optional[torch.Tensor]:
+                     sinks: Optional[torch.Tensor] = None, leave_chunks: bool = False, softcap: float = 0.0,
+                     bias: Optional[torch.Tensor] = None, keep_first: int = 0) -> Optional[torch.Tensor]:
     """The same attention for single query tokens, split over the keys, on the matrix cores
     (bfloat16, head_dim a multiple of 16 up to 128, group size <= 16, page size a multiple of 8).
     ``max_keys`` is an upper bound of the keys any listed token sees (its position + 1), known on
     the host; it only sizes the launch.  ``leave_chunks`` (with ``sinks``, without a token list): nothing is merged
-    or written to ``out``; every token's chunks stay in ``workspace`` for ``attention_decode_project``."""
+    or written to ``out``; every token's chunks stay in ``workspace`` for ``attention_decode_project``.
+    ``softcap``, ``bias`` (float32 [nh, L]) and ``keep_first``: scores are capped as cap * tanh(score / cap), then
+    take ``bias[head, min(distance, L - 1)]``; the sequence's first ``keep_first`` positions stay visible beside the
+    window."""
     out, n, count, ldq, ldo, pages, ps = _attention_args("attention_decode", q, kcache, vcache, tok_seq, tok_pos,
                                                          block_tables, nh, nkv, d, tok_index,
                                                          q if (leave_chunks and out is None) else out)   # (nothing is written there)
@@ -439,7 +459,13 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
             _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
             nh, nkv, d, ps, int(window), float(scale), max_chunks, _p(workspace),
             workspace.numel() if workspace is not None else 0)
-    if sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
+    extras = _score_extras("attention_decode", nh, q, softcap, bias, keep_first)
+    if extras is not None:
+        if leave_chunks:
+            raise ValueError("attention_decode: capped or biased scores are merged here")
+        _lib.call("zi_attention_decode_biased", *args,
+                  _p(_sinks(sinks, nh, q, "attention_decode") if sinks is not None else None), *extras, _stream())
+    elif sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
         _lib.call("zi_attention_decode_sink", *args, _p(_sinks(sinks, nh, q, "attention_decode")), _stream())
     else:
         _lib.call("zi_attention_decode", *args, _stream())
@@ -736,7 +762,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
                       workspace: Optional[torch.Tensor] = None, tile: int = 0, alone: bool = False,
-                      sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      sinks: Optional[torch.Tensor] = None, softcap: float = 0.0, bias: Optional[torch.Tensor] = None,
+                      keep_first: int = 0) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
@@ -748,7 +775,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     cut over several workgroups and merged, which needs ``workspace`` (``attention_prefill_workspace``
     entries of float32; allocated here when not given).  A bound that is too low leaves NaN in the rows
     concerned.  ``alone`` (where the head size has tiles of 128): workgroups of four wavefronts, two to a compute
-    unit, which pays for launches of many tiles; the result differs by rounding."""
+    unit, which pays for launches of many tiles; the result differs by rounding.  ``softcap``, ``bias`` and
+    ``keep_first`` as for ``attention_decode``; with any of them tiles hold ``attention_prefill_tile_min()`` queries."""
     _gpu("attention_prefill", q, kcache, vcache, tile_entry, tile_off, entry_start, entry_len, entry_past,
          block_tables, out)
     ldq, wq = _rows(q, "attention_prefill q")
@@ -791,7 +819,13 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
             _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
             max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), int(bool(alone)),
             chunk_keys)
-    if sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
+    extras = _score_extras("attention_prefill", nh, q, softcap, bias, keep_first)
+    if extras is not None:
+        if tile != attention_prefill_tile_min() or alone:
+            raise ValueError("attention_prefill: capped or biased scores take the smallest tiles")
+        _lib.call("zi_attention_prefill_biased", *args,
+                  _p(_sinks(sinks, nh, q, "attention_prefill") if sinks is not None else None), *extras, _stream())
+    elif sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
         _lib.call("zi_attention_prefill_sink", *args, _p(_sinks(sinks, nh, q, "attention_prefill")), _stream())
     else:
         _lib.call("zi_attention_prefill", *args, _stream())

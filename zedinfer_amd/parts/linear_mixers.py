@@ -23,7 +23,7 @@ from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
 from .base import MIXERS, KVCacheRequest, LayerMemory, Mixer, Runtime, StateRequest, register_mixer
-from .mixers import attention_cache_request
+from .mixers import LONG_TILE, attention_cache_request, attention_planner
 from .rows import ProductRows
 
 
@@ -268,6 +268,38 @@ class BiasedWindowAttention(ProjectedMixer):
         self.bias = distance_bias_table(weights["rel"], float(p["bias_max"])) if "rel" in weights else None
         self.state_floats = 0
         self.init_shift(spec, weights)
+        # the step's tokens are dealt out as for any softmax attention: single tokens, tiles of prompt portions
+        self.plan_key = attention_planner(LONG_TILE, self.nh).key
+
+    def planner(self):
+        return attention_planner(LONG_TILE, self.nh)
+
+    def attend(self, q, att, batch, view, kc, vc) -> None:
+        """Tokens of short entries go to the kernel that splits one query's keys over many wavefronts, longer
+        portions to the matrix-core prompt kernel, both with the cap, the bias and the kept positions; every shape
+        those kernels do not take (float32, heads beyond 128) goes to the plain kernel."""
+        extras = dict(softcap=self.softcap, bias=self.bias, keep_first=self.keep_first)
+        plan = batch.plans[self.plan_key]
+        n_short, n_long, N = plan.sizes["num_short"], plan.sizes["num_long"], batch.num_tokens
+        cores = (ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2])
+                 and ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2]))
+        if not cores:
+            ops.attention_biased(q, kc, vc, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
+                                 self.scale, self.window, out=att, **extras)
+            return
+        if n_short:
+            ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n_short, self.nh, self.d),), torch.float32)
+            ops.attention_decode(q, kc, vc, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
+                                 self.scale, plan.sizes["max_short_keys"], self.window, out=att,
+                                 tok_index=plan.dev["short_idx"] if n_short < N else None, workspace=ws, **extras)
+        if n_long:
+            max_keys = plan.sizes["max_long_keys"]
+            need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, max_keys, self.window, plan.sizes["num_tiles"])
+            ws = self.rt.buffer("attn_prompt_split", (need,), torch.float32) if need else None
+            ops.attention_prefill(q, kc, vc, plan.dev["tile_entry"], plan.dev["tile_off"], batch.entry_start,
+                                  batch.entry_len, batch.entry_past, view.block_tables, self.nh, self.nkv, self.d,
+                                  self.scale, self.window, out=att, max_keys=max_keys, workspace=ws,
+                                  tile=plan.sizes["tile"], **extras)
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         if self.window > 0:
@@ -285,9 +317,7 @@ class BiasedWindowAttention(ProjectedMixer):
                             vc if memory.writes else None, self.nh, self.nkv, self.dim, self.vdim, self.d, self.eps,
                             norm_values=self.value_norm)
         att = rt.buffer("attn_out", (n, self.nh * self.d))
-        ops.attention_biased(q, kc, vc, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
-                             self.scale, self.window, out=att, softcap=self.softcap, bias=self.bias,
-                             keep_first=self.keep_first)
+        self.attend(q, att, batch, view, kc, vc)
         g_at = qd + kd + self.nkv * self.vdim
         ops.gate_heads(att, proj[:, g_at:g_at + self.nh * self.vdim], self.vdim, self.d, "sigmoid", out=y, scale=scale)
 
