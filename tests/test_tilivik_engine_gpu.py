@@ -177,23 +177,25 @@ def _sharp_config(window, keep, cap):
 
 
 def _sharp_weights(cfg):
-    """Token 5 is the only one whose key points where every query points (a score of 40 against 0 before the cap),
-    and its value is the only one with a large first entry."""
+    """Token 5 is the only one with a large first channel; the key's first dim reads that channel, every query's
+    first dim reads the last channel, which the sinusoid holds near 1 at every position: the marked key scores about
+    20 against at most 5 for the others, and its value is the only one that is large on the dim that the output
+    matrix lets through four-fold."""
     w = {k: torch.zeros_like(v) for k, v in models.make_weights(cfg, 0).items()}
     W, V = cfg["width"], cfg["vocab"]
     g = torch.Generator().manual_seed(3)
     w["embed"] = 0.3 * torch.randn(V, W, generator=g)
     w["embed"][:, 0] = 0.0
-    w["embed"][5, 0] = 6.0                                    # the mark of the far token
+    w["embed"][:, W - 1] = 0.0
+    w["embed"][5, 0] = 6.0                                    # the mark
     w["l0.norm1"], w["final.norm"] = torch.tensor(1.0), torch.tensor(1.0)
     w["l0.mix.right.norm"] = torch.ones(8)
-    w["l0.mix.left.k"][0, 0] = 10.0                           # the key's dim 0 is the mark
-    w["l0.mix.left.q"][0] = 0.0
-    w["l0.mix.left.q"][0, 1:] = 0.05 * torch.randn(W - 1, generator=g).abs() + 0.4     # every query has about 4 on dim 0
-    w["l0.mix.left.q"][32] = w["l0.mix.left.q"][0]
-    w["l0.mix.left.v"][0, 0] = 1.0                            # the value's dim 0 is the mark as well
-    w["l0.mix.left.v"][1, 1:] = 0.3                           # and every value has something on dim 1
-    w["l0.mix.left.o"][0, 0], w["l0.mix.left.o"][1, 33] = 1.0, 1.0
+    w["l0.mix.left.k"][0, 0] = 1.0
+    w["l0.mix.left.q"][0, W - 1] = 3.0
+    w["l0.mix.left.q"][32, W - 1] = 3.0
+    w["l0.mix.left.v"][0, 0] = 1.0
+    w["l0.mix.left.v"][1, 1:] = 0.3                           # every value has something on dim 1
+    w["l0.mix.left.o"][0, 0], w["l0.mix.left.o"][1, 33] = 4.0, 1.0
     w["head"] = 0.2 * torch.randn(V, W, generator=g)
     return w
 
@@ -235,11 +237,11 @@ def test_a_marked_key_at_the_edge_of_the_window_and_of_the_kept_positions(tmp_pa
     other[at] = 6
     moved = (ref_model.forward(other).float()[rows] - ref[rows]).abs().amax(dim=1)
     if where == "window_in":
-        assert float(moved[-1]) > 0.1 * scale
+        assert float(moved.min()) > 0.08 * scale
     elif where == "window_out":
-        assert float(moved[1:].max()) < 1e-3 * scale and float(moved[0]) > 0.1 * scale      # T - 40 still sees it
+        assert float(moved[1:].max()) < 1e-3 * scale and float(moved[0]) > 0.08 * scale      # T - 40 still sees it
     elif where == "kept_in":
-        assert float(moved.min()) > 0.1 * scale
+        assert float(moved.min()) > 0.08 * scale
     else:
         assert float(moved.max()) < 1e-3 * scale
 

@@ -91,8 +91,9 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
     constexpr int DP = la_place(D);               // floats of a staged row
     constexpr int NSEG = GATED ? 3 : 2;           // k, q (, decay)
     constexpr int THREADS = LA_WAVES * ZI_WAVE;
-    constexpr int NE = TC * NSEG * D;
-    constexpr int PRE = (NE + THREADS - 1) / THREADS;
+    constexpr int PSEG = TC * D / THREADS;        // values of k (or q, or the decay) of a chunk a thread stages
+    constexpr int PRE = NSEG * PSEG;
+    static_assert(PSEG * THREADS == TC * D, "a chunk's rows divide evenly over the threads");
     static_assert(TC <= LA_PARTS && TC * LA_WCOLS <= THREADS, "a chunk's read-outs are written by the lanes of a row");
     __shared__ __attribute__((aligned(16))) float rows[2][TC][NSEG][DP];
     __shared__ float vs[2][TC][LA_WCOLS];
@@ -120,42 +121,43 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
     float pre[PRE], vpre;
     unsigned ok_bits = 0;
     bool v_ok = false;
-    auto fetch = [&](int base) {
+    auto fetch = [&](int base) __attribute__((always_inline)) {
         const int n_in = len - base;      // tokens of the chunk (more than TC: all TC; none or fewer past the end)
         const int tb = t0 + (base < len ? base : len - 1);
         ok_bits = 0;
 #pragma unroll
-        for (int i = 0; i < PRE; ++i) {
-            const int idx = i * THREADS + tid;
-            const int tt = idx / (NSEG * D), rem = idx % (NSEG * D), seg = rem / D, d = rem % D;
-            const bool ok = idx < NE && tt < n_in && d < dim;
-            const int64_t tok = tb + (ok ? tt : 0);
-            const int dd = ok ? d : 0;
+        for (int seg = 0; seg < NSEG; ++seg) {      // which array a pass reads is known when the loop is unrolled
             const float* src = seg == 0 ? k : (seg == 1 ? q : decay);
-            pre[i] = src[tok * (seg == 2 ? ld_decay : ld) + qk_at + dd];
-            ok_bits |= (unsigned)ok << i;
+            const int64_t stride = seg == 2 ? ld_decay : ld;
+#pragma unroll
+            for (int u = 0; u < PSEG; ++u) {
+                const int idx = u * THREADS + tid, tt = idx / D, d = idx % D;
+                const bool ok = tt < n_in && d < dim;
+                pre[seg * PSEG + u] = src[(int64_t)(tb + (ok ? tt : 0)) * stride + qk_at + (ok ? d : 0)];
+                ok_bits |= (unsigned)ok << (seg * PSEG + u);
+            }
         }
         const int tt = tid / LA_WCOLS, cc = tid % LA_WCOLS;
         v_ok = tid < TC * LA_WCOLS && tt < n_in && col0 + cc < vdim;
         vpre = v[(int64_t)(tb + (v_ok ? tt : 0)) * ld + v_at + (v_ok ? col0 + cc : 0)];
     };
-    auto stash = [&](int b) {
+    auto stash = [&](int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < PRE; ++i) {
-            const int idx = i * THREADS + tid;
-            if (idx >= NE) continue;
-            const int tt = idx / (NSEG * D), rem = idx % (NSEG * D), seg = rem / D, d = rem % D;
-            float x = ((ok_bits >> i) & 1u) ? pre[i] : 0.f;
-            if (seg < 2 && act) x = la_silu(x);
-            if (seg == 1) x *= qscale;
-            rows[b][tt][seg][la_place(d)] = x;
-        }
+        for (int seg = 0; seg < NSEG; ++seg)
+#pragma unroll
+            for (int u = 0; u < PSEG; ++u) {
+                const int idx = u * THREADS + tid, tt = idx / D, d = idx % D;
+                float x = ((ok_bits >> (seg * PSEG + u)) & 1u) ? pre[seg * PSEG + u] : 0.f;
+                if (seg < 2 && act) x = la_silu(x);
+                if (seg == 1) x *= qscale;
+                rows[b][tt][seg][la_place(d)] = x;
+            }
         if (tid < TC * LA_WCOLS) {
             const float x = v_ok ? vpre : 0.f;
             vs[b][tid / LA_WCOLS][tid % LA_WCOLS] = act ? la_silu(x) : x;
         }
     };
-    auto work = [&](int base, int b) {
+    auto work = [&](int base, int b) __attribute__((always_inline)) {
         const int n_in = len - base;
         float accs[TC];
 #pragma unroll
@@ -165,17 +167,24 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
                 float kk[R], qq[R], aa[R];
                 const float* kr = &rows[b][tt][0][la_place(p * R)];
                 const float* qr = &rows[b][tt][1][la_place(p * R)];
+                const float* ar = &rows[b][tt][NSEG - 1][la_place(p * R)];
                 if constexpr (R == 2) {
-                    *reinterpret_cast<float2*>(kk) = *reinterpret_cast<const float2*>(kr);
-                    *reinterpret_cast<float2*>(qq) = *reinterpret_cast<const float2*>(qr);
-                    if constexpr (GATED) *reinterpret_cast<float2*>(aa) = *reinterpret_cast<const float2*>(&rows[b][tt][NSEG - 1][la_place(p * R)]);
+                    const float2 k2 = *reinterpret_cast<const float2*>(kr), q2 = *reinterpret_cast<const float2*>(qr);
+                    kk[0] = k2.x; kk[1] = k2.y; qq[0] = q2.x; qq[1] = q2.y;
+                    if constexpr (GATED) {
+                        const float2 a2 = *reinterpret_cast<const float2*>(ar);
+                        aa[0] = a2.x; aa[1] = a2.y;
+                    }
                 } else {
 #pragma unroll
                     for (int r4 = 0; r4 < R; r4 += 4) {
-                        *reinterpret_cast<float4*>(kk + r4) = *reinterpret_cast<const float4*>(kr + r4);
-                        *reinterpret_cast<float4*>(qq + r4) = *reinterpret_cast<const float4*>(qr + r4);
-                        if constexpr (GATED)
-                            *reinterpret_cast<float4*>(aa + r4) = *reinterpret_cast<const float4*>(&rows[b][tt][NSEG - 1][la_place(p * R)] + r4);
+                        const float4 k4 = *reinterpret_cast<const float4*>(kr + r4), q4 = *reinterpret_cast<const float4*>(qr + r4);
+                        kk[r4] = k4.x; kk[r4 + 1] = k4.y; kk[r4 + 2] = k4.z; kk[r4 + 3] = k4.w;
+                        qq[r4] = q4.x; qq[r4 + 1] = q4.y; qq[r4 + 2] = q4.z; qq[r4 + 3] = q4.w;
+                        if constexpr (GATED) {
+                            const float4 a4 = *reinterpret_cast<const float4*>(ar + r4);
+                            aa[r4] = a4.x; aa[r4 + 1] = a4.y; aa[r4 + 2] = a4.z; aa[r4 + 3] = a4.w;
+                        }
                     }
                 }
                 const float vv = vs[b][tt][wave * LA_COLS + c];
