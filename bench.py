@@ -449,7 +449,7 @@ def tilivik_shape(size, layers, vocab):
         right = dict(heads=z["heads"] // 2, dim=64, vdim=128, tau=16.0, rank=16)
         out.append(dict(type="parallel", mlp=mlp, mixer=dict(left=left, right=right, left_scale=0.7, right_scale=0.7)))
     cfg = dict(architecture="Tilivik", width=z["width"], vocab=vocab, norm=dict(eps=1e-6),
-               embedding=dict(bigram=dict(buckets=65521, mul_prev=31, mul_cur=17)), layers=out)
+               embedding=dict(bigram=dict(buckets=65521, mul_prev=257, mul_cur=263)), layers=out)
     if layers > held:
         cfg["loop"] = dict(start=1, stop=3, times=1 + (layers - held) // 2)
     return cfg

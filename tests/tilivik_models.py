@@ -196,8 +196,8 @@ def random_config(seed):
     cfg = dict(architecture="Tilivik", width=width, vocab=rng.choice([97, 256, 411]),
                norm=dict(eps=rng.choice([1e-6, 1e-5, 3e-6])), layers=[])
     if rng.random() < 0.75:
-        cfg["embedding"] = dict(bigram=dict(buckets=rng.choice([7, 101, 509]), mul_prev=rng.choice([1, 3, 31, 1009]),
-                                            mul_cur=rng.choice([1, 5, 17])))
+        cfg["embedding"] = dict(bigram=dict(buckets=rng.choice([7, 101, 509]), mul_prev=rng.choice([1, 3, 29, 1009]),
+                                            mul_cur=rng.choice([1, 5, 19])))
     n_layers = rng.randint(2, 5)
     for i in range(n_layers):
         r = rng.random()
