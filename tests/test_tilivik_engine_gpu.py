@@ -246,6 +246,41 @@ def test_a_marked_key_at_the_edge_of_the_window_and_of_the_kept_positions(tmp_pa
         assert float(moved.max()) < 1e-3 * scale
 
 
+LONG = dict(
+    architecture="Tilivik", width=128, vocab=180, norm=dict(eps=1e-6),
+    embedding=dict(bigram=dict(buckets=251, mul_prev=5, mul_cur=3)),
+    layers=[dict(type="parallel", mlp=dict(kind="moe", expert=dict(ff=32), router=dict(experts=4, top=2)),
+                 mixer=dict(left=dict(heads=4, kv_heads=2, dim=64, vdim=64, scale=0.125, softcap=12.0, bias_max=3000, bias_rows=16,
+                                      mask=dict(size=2200, keep_first=3)),
+                            left_scale=0.9, right=dict(heads=2, dim=16, vdim=32, tau=32.0, rank=4), right_scale=0.8))])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whose_keys_are_cut_over_workgroups(tmp_path, dtype):
+    """2,300 tokens under a window of 2,200 in two portions and a few decoded tokens: tiles whose keys are cut over
+    several workgroups and merged, tokens whose keys are more than one chunk, the window passing the kept positions."""
+    from zedinfer_amd.engine import StepEntry
+    cfg = LONG
+    T = 2300
+    toks = traces.random_tokens(cfg["vocab"], T, seed=4)
+    folder = models.write_config(str(tmp_path / "long"), cfg,
+                                 models.make_weights(cfg, 2, torch.float32 if dtype == "float32" else torch.bfloat16))
+    ref = plain.PlainTilivik.from_folder(folder).forward(toks).float()
+    engine = _engine(folder, dtype, pages=160, page=16)
+    seq = engine.open("x")
+    rows = [5, 900, 999]
+    out = [engine.step([StepEntry(seq, toks[:1000], rows)]).cpu()]
+    more = [0, 1100, 1202, 1203, 1289]                      # positions 1000 .. 2289
+    out.append(engine.step([StepEntry(seq, toks[1000:2290], more)]).cpu())
+    rows += [1000 + m for m in more]
+    for t in range(2290, T):
+        out.append(engine.step([StepEntry(seq, [toks[t]], [0])]).cpu())
+        rows.append(t)
+    engine.close(seq)
+    err = (torch.cat(out).double() - ref[rows].double()).abs()
+    _rows_within(err.amax(dim=1).numpy(), err.mean(dim=1).numpy(), float(ref.abs().max()), dtype, "long prompt")
+
+
 @pytest.mark.parametrize("name", ["main", "odd"])
 def test_greedy_generation_through_the_serving_engine(tmp_path, name):
     """Several requests at once through InferenceEngine (its scheduler cuts the prompts into portions of 16 tokens and
