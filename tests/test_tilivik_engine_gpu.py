@@ -246,6 +246,36 @@ def test_a_marked_key_at_the_edge_of_the_window_and_of_the_kept_positions(tmp_pa
         assert float(moved.max()) < 1e-3 * scale
 
 
+# models of one kind of layer only: no pages at all (nothing but state), and nothing but pages and state of one layer
+ONLY_LINEAR = dict(
+    architecture="Tilivik", width=64, vocab=90, norm=dict(eps=1e-6), loop=dict(start=0, stop=2, times=2),
+    layers=[dict(type="lightning", mixer=dict(heads=2, dim=16, vdim=32, decay=[0.9, 1.0]), mlp=None),
+            dict(type="lightning", mixer=dict(heads=4, dim=8, vdim=16, decay=[0.5, 0.7, 0.9, 0.99]),
+                 mlp=dict(kind="moe", expert=dict(ff=24), router=dict(experts=3, top=1)))])
+ONLY_SOFTMAX = dict(
+    architecture="Tilivik", width=64, vocab=90, norm=dict(eps=1e-6), embedding=dict(bigram=dict(buckets=2, mul_prev=1, mul_cur=2)),
+    layers=[dict(type="parallel", mlp=None,
+                 mixer=dict(left=dict(heads=2, kv_heads=2, dim=32, vdim=32, scale=0.2), left_scale=1.0,
+                            right=dict(heads=1, dim=8, vdim=8, tau=2.0, rank=1), right_scale=1.0))])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["only_linear", "only_softmax"])
+def test_models_of_one_kind_of_layer(tmp_path, which, dtype):
+    cfg = ONLY_LINEAR if which == "only_linear" else ONLY_SOFTMAX
+    requests = {f"o{i}": traces.random_tokens(cfg["vocab"], n, seed=30 + i) for i, n in enumerate([50, 3, 77, 20, 9])}
+    folder = models.write_config(str(tmp_path / which), cfg,
+                                 models.make_weights(cfg, 6, torch.float32 if dtype == "float32" else torch.bfloat16))
+    ref_model = plain.PlainTilivik.from_folder(folder)
+    ref = {rid: ref_model.forward(toks).float() for rid, toks in requests.items()}
+    engine = _engine(folder, dtype, pages=40, page=8, max_live=3)
+    assert len(engine.cache.groups) == (0 if which == "only_linear" else 1)
+    for what, steps in (("mixed", traces.mixed(requests, max_live=3, seed=2)), ("whole", traces.whole(requests)),
+                        ("portions", traces.portions(requests, seed=5, sizes=(2, 9, 1, 4)))):
+        out = traces.run_in_process(engine, steps)
+        _check(steps, out, ref, dtype, (which, what))
+
+
 LONG = dict(
     architecture="Tilivik", width=128, vocab=180, norm=dict(eps=1e-6),
     embedding=dict(bigram=dict(buckets=251, mul_prev=5, mul_cur=3)),
