@@ -111,6 +111,11 @@ class ProjectedMixer(Mixer):
         state = memory.state[:, at:at + self.state_floats] if self.state_floats else None
         self.mix(proj, batch, memory, state, y, 1.0)
         if out is None:
+            if ops.linear_sums_supported(y, self.w_out):
+                # few rows: the product's partial sums go on as they are; the norm (or the step between layers) that
+                # takes the mixer's result adds them, so no kernel is launched for that alone
+                S = ops.linear_splits(n, self.hidden, self.w_out.shape[1])
+                return ops.linear_sums(y, self.w_out, out=rt.buffer("mix_out_sums", (S, n, self.hidden), torch.float32))
             out = rt.buffer("mix_out", (n, self.hidden), torch.float32)
         return ops.linear(y, self.w_out, out=out)
 
