@@ -70,7 +70,7 @@ struct DecProjection {
 
 // exp2-based tanh: 1 - 2 / (2^(2 x log2 e) + 1), right at both ends
 __device__ __forceinline__ float dec_tanh(float x) {
-    return 1.f - 2.f / (__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
 }
 
 // BIASED: the scores are capped and biased by distance, and the sequence's first positions stay visible beside the
@@ -479,7 +479,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                     if (ex.softcap > 0.f) sc = ex.softcap * dec_tanh(sc * inv_cap);
                     if (brow) {
                         int dist = p - key;
-                        dist = dist < 0 ? 0 : (dist < ex.bias_len ? dist : ex.bias_len - 1);
+                        dist = (int)min((unsigned)dist, (unsigned)(ex.bias_len - 1));      // (a key ahead of the query is masked anyway)
                         sc += brow[dist];
                     }
                     sc *= 1.4426950408889634f;

@@ -35,6 +35,7 @@
 #include "zi_common.h"
 #include "zi_api.h"
 #include "zi_paging.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4_t;
@@ -63,7 +64,7 @@ __device__ __forceinline__ uint4 pf_keep(uint4 v, int keep) {
 
 // exp2-based tanh: 1 - 2 / (2^(2 x log2 e) + 1), right at both ends (2^inf = inf gives 1, 2^-inf = 0 gives -1)
 __device__ __forceinline__ float pf_tanh(float x) {
-    return 1.f - 2.f / (__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.8853900817779268f) + 1.f);
 }
 
 // BIASED: the scores are capped and biased by distance, and the sequence's first positions stay visible beside the
@@ -262,26 +263,34 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         const bool whole = !BIASED && kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
         float mx = -INFINITY;
         if constexpr (BIASED) {
-            // every score becomes its capped and biased value, in base-2 units already
+            // every score becomes its capped and biased value, in base-2 units already; a block that every query of
+            // the wavefront sees whole needs no mask here either
             const float inv_cap = ex.softcap > 0.f ? 1.f / ex.softcap : 0.f;
             const float* brow = ex.bias ? ex.bias + (int64_t)h * ex.bias_len : nullptr;
+            auto transform = [&](auto masked) __attribute__((always_inline)) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
-                    const bool vis = key <= qpos && (window <= 0 || key > qpos - window || key < ex.keep_first);
-                    float sc = s[t][x] * scale;
-                    if (ex.softcap > 0.f) sc = ex.softcap * pf_tanh(sc * inv_cap);
-                    if (brow) {
-                        int dist = qpos - key;
-                        dist = dist < 0 ? 0 : (dist < ex.bias_len ? dist : ex.bias_len - 1);
-                        sc += brow[dist];
+                    for (int x = 0; x < 4; ++x) {
+                        const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                        float sc = s[t][x] * scale;
+                        if (ex.softcap > 0.f) sc = ex.softcap * pf_tanh(sc * inv_cap);
+                        if (brow) {
+                            int dist = qpos - key;
+                            dist = (int)min((unsigned)dist, (unsigned)(ex.bias_len - 1));      // (a key ahead of the query is masked anyway)
+                            sc += brow[dist];
+                        }
+                        float v = sc * 1.4426950408889634f;
+                        if constexpr (decltype(masked)::value) {
+                            const bool vis = key <= qpos && (window <= 0 || key > qpos - window || key < ex.keep_first);
+                            v = vis ? v : -INFINITY;
+                        }
+                        s[t][x] = v;
+                        mx = fmaxf(mx, v);
                     }
-                    const float v = vis ? sc * 1.4426950408889634f : -INFINITY;
-                    s[t][x] = v;
-                    mx = fmaxf(mx, v);
-                }
+            };
+            if (kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window)) transform(std::false_type{});
+            else transform(std::true_type{});
         } else if (whole) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
