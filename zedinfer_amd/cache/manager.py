@@ -52,14 +52,20 @@ class CacheGroup:
     pool: PagePool
     caches: Dict[int, KVCacheRequest] = field(default_factory=dict)    # cache id -> what its layer asked for
     keep_first: int = 0            # a window group keeps the pages of positions below this as well
+    stride: int = 1                # positions a row of the cache stands for (more than 1: summaries of blocks)
 
     @property
     def kept_pages(self) -> int:
         """Logical pages at the start of a sequence that a window group never gives back early."""
         return self.pages_for(self.keep_first) if self.kind == "window" else 0
 
+    def rows_for(self, tokens: int) -> int:
+        """Rows of the cache that a sequence of ``tokens`` tokens has written: one a position, or one for every whole
+        block of ``stride`` positions."""
+        return tokens if self.stride == 1 else tokens // self.stride
+
     def pages_for(self, tokens: int) -> int:
-        return (tokens + self.page_size - 1) // self.page_size
+        return (self.rows_for(tokens) + self.page_size - 1) // self.page_size
 
     def promise_for(self, tokens: int, max_step_tokens: int) -> int:
         """Most pages a sequence of ``tokens`` tokens holds at once in this group."""
@@ -116,18 +122,25 @@ class CacheManager:
         self.device = torch.device(device) if device is not None else None
         self.groups: List[CacheGroup] = []
         self.group_of_cache: Dict[int, int] = {}
-        keys: Dict[Tuple[str, int, int], int] = {}
-        for cid in sorted(kv_requests):
+        keys: Dict[Tuple[str, int, int, int], int] = {}
+        # (a mixer's further caches stand under (cache id, name): after the layers' own)
+        for cid in sorted(kv_requests, key=lambda c: (1, c[0], str(c[1])) if isinstance(c, tuple) else (0, c, "")):
             rq = kv_requests[cid]
             if rq.kind not in ("full", "window") or (rq.kind == "window" and rq.window <= 0):
                 raise ValueError(f"cache {cid}: unknown cache kind {rq.kind!r} / window {rq.window}")
             if rq.keep_first < 0:
                 raise ValueError(f"cache {cid}: negative keep_first")
-            key = (rq.kind, rq.window if rq.kind == "window" else 0, rq.keep_first if rq.kind == "window" else 0)
+            stride = int(getattr(rq, "stride", 1) or 1)
+            if stride < 1 or (stride > 1 and rq.kind != "full"):
+                raise ValueError(f"cache {cid}: a cache of one row for every {stride} positions must keep all of them")
+            key = (rq.kind, rq.window if rq.kind == "window" else 0, rq.keep_first if rq.kind == "window" else 0, stride)
             if key not in keys:
                 keys[key] = len(self.groups)
-                self.groups.append(CacheGroup(rq.kind, key[1], self.page_size, PagePool(self.num_pages),
-                                              keep_first=key[2]))
+                # rows for every so many positions need that many fewer pages, and one more a request for the page
+                # each has begun
+                pages = self.num_pages if stride == 1 else -(-self.num_pages // stride) + self.max_requests
+                self.groups.append(CacheGroup(rq.kind, key[1], self.page_size, PagePool(pages),
+                                              keep_first=key[2], stride=stride))
             g = keys[key]
             self.groups[g].caches[cid] = rq
             self.group_of_cache[cid] = g
@@ -138,7 +151,7 @@ class CacheManager:
         self.state_requests = dict(state_requests)
         if self.device is not None:
             for cid, rq in kv_requests.items():
-                self.tensors[cid] = {name: torch.zeros((self.num_pages,) + pt.page_shape(self.page_size),
+                self.tensors[cid] = {name: torch.zeros((self.groups[self.group_of_cache[cid]].pool.total,) + pt.page_shape(self.page_size),
                                                        dtype=pt.dtype or dtype, device=self.device)
                                      for name, pt in rq.tensors}
             for cid, sr in state_requests.items():
@@ -165,8 +178,10 @@ class CacheManager:
         out.embedding = LayerMemory(state=self.state.get(EMBEDDING_CACHE))
         for st in schedule:
             g = self.group_of_cache.get(st.cache, -1)
+            sides = {cid[1]: LayerMemory(group=gi, tensors=self.tensors.get(cid, {}), writes=st.writes_cache)
+                     for cid, gi in self.group_of_cache.items() if isinstance(cid, tuple) and cid[0] == st.cache}
             out.append(LayerMemory(group=g, tensors=self.tensors.get(st.cache, {}), writes=st.writes_cache,
-                                   state=self.state.get(st.cache)))
+                                   state=self.state.get(st.cache), sides=sides))
         return out
 
     # ---- admission ---------------------------------------------------------------
@@ -224,7 +239,8 @@ class CacheManager:
         try:
             for gi, g in enumerate(self.groups):
                 table = seq.pages[gi]
-                last = (new_len - 1) // g.page_size if new_len > 0 else -1
+                rows = g.rows_for(new_len)
+                last = (rows - 1) // g.page_size if rows > 0 else -1
                 if len(table) <= last:
                     if growth is None:
                         growth = Growth(taken=[], grown=[0] * len(self.groups), old_lens=[len(t) for t in seq.pages])
@@ -298,6 +314,17 @@ class CacheManager:
         g = self.groups[group]
         pos = np.arange(start, start + count, dtype=np.int64)
         table = np.asarray(seq.pages[group], dtype=np.int64)
+        if g.stride > 1:
+            # a row for every `stride` positions: the slot of the row that a position completes, -1 for the others
+            ends = (pos + 1) % g.stride == 0
+            rows = pos // g.stride
+            out = np.full(count, -1, dtype=np.int64)
+            if ends.any():
+                pages = table[rows[ends] // g.page_size]
+                if (pages < 0).any():
+                    raise RuntimeError(f"request {seq.request_id!r}: a block ending in [{start}, {start + count}) has no page")
+                out[ends] = pages * g.page_size + rows[ends] % g.page_size
+            return out.astype(np.int32)
         pages = table[pos // g.page_size]
         if (pages < 0).any():
             raise RuntimeError(f"request {seq.request_id!r}: a position in [{start}, {start + count}) has no page")

@@ -506,3 +506,99 @@ class TilivikConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+@dataclass(frozen=True)
+class KegozenConfig(ModelConfig):
+    """The Kegozen design's config.json: ``width``, ``vocab``, ``norm.eps`` and a list ``layers`` whose entries each
+    name a mixer by ``type`` ("mamba2": a selective state-space mixer; "attention": grouped-query attention under a
+    sliding window that sees older positions as means of blocks; "latent_attention": causal attention whose queries,
+    keys and values come through latents) with its sizes and constants under ``mixer``, and a feed-forward under
+    ``mlp`` (``kind`` "dense" with ``ff``; ``kind`` "moe" with ``router.experts`` / ``router.top``, ``expert.ff`` and
+    optionally ``shared.ff``; or null for none).  Every size and constant of a model is read from here; the shared keys
+    of ``ModelConfig`` that the format does not have keep their neutral values."""
+
+    layers: Tuple[Any, ...] = ()
+    norm_eps: float = 1e-6
+
+    MIXER_KEYS = {"mamba2": ("heads", "vdim", "state", "groups", "conv", "norm_groups"),
+                  "attention": ("heads", "kv_heads", "dim", "vdim", "scale"),
+                  "latent_attention": ("heads", "dim", "rot_dim", "vdim", "kv_rank", "scale")}
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "KegozenConfig":
+        missing = [k for k in ("width", "vocab", "layers", "norm") if k not in d]
+        if missing:
+            raise ConfigError("config.json lacks required key(s): " + ", ".join(missing))
+        if not isinstance(d["layers"], (list, tuple)) or not d["layers"]:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        if not isinstance(d["norm"], Mapping) or "eps" not in d["norm"]:
+            raise ConfigError("config.json: 'norm' must give 'eps'")
+        eos = d.get("eos_token_id")
+        cfg = cls(architectures=(str(d.get("architecture", "Kegozen")),), model_type="kegozen",
+                  torch_dtype=str(d.get("torch_dtype") or "bfloat16"), hidden_size=_as_int(d, "width"),
+                  vocab_size=_as_int(d, "vocab"), num_hidden_layers=len(d["layers"]),
+                  eos_token_ids=() if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos])),
+                  layers=tuple(json.loads(json.dumps(layer)) for layer in d["layers"]), norm_eps=float(d["norm"]["eps"]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.hidden_size <= 0 or self.vocab_size <= 0:
+            raise ConfigError("config.json: 'width' and 'vocab' must be positive")
+        if not (self.norm_eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.norm_eps}")
+        for i, layer in enumerate(self.layers):
+            kind = layer.get("type") if isinstance(layer, Mapping) else None
+            if kind not in self.MIXER_KEYS:
+                raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
+            m = layer.get("mixer")
+            lacking = [k for k in self.MIXER_KEYS[kind] if not isinstance(m, Mapping) or k not in m]
+            if lacking:
+                raise ConfigError(f"config.json: layer {i} ({kind}) lacks mixer key(s): " + ", ".join(lacking))
+            if any(int(m[k]) <= 0 for k in self.MIXER_KEYS[kind] if k != "scale") or ("scale" in m and not float(m["scale"]) > 0):
+                raise ConfigError(f"config.json: layer {i} ({kind}): sizes and the scale must be positive")
+            if kind == "mamba2":
+                if int(m["heads"]) % int(m["groups"]) or (int(m["heads"]) * int(m["vdim"])) % int(m["norm_groups"]):
+                    raise ConfigError(f"config.json: layer {i}: heads must be a multiple of groups, heads * vdim of norm_groups")
+            else:
+                rot = m.get("rot")
+                if rot is not None and (not isinstance(rot, Mapping) or "base" not in rot or "dims" not in rot
+                                        or int(rot["dims"]) % 2 or int(rot["dims"]) <= 0 or not float(rot["base"]) > 1):
+                    raise ConfigError(f"config.json: layer {i}: rot needs a base above 1 and an even, positive dims")
+            if kind == "attention":
+                if int(m["heads"]) % int(m["kv_heads"]):
+                    raise ConfigError(f"config.json: layer {i}: heads must be a multiple of kv_heads")
+                if m.get("rot") is not None and (int(m["rot"]["dims"]) > int(m["dim"]) or int(m["vdim"]) % 2):
+                    raise ConfigError(f"config.json: layer {i}: rot.dims within dim, and an even vdim")
+                mask = m.get("mask")
+                if mask is not None and (not int(mask.get("size", 0)) > 0 or int(mask.get("pool", 0) or 0) < 0):
+                    raise ConfigError(f"config.json: layer {i}: mask.size must be positive, mask.pool not negative")
+            if kind == "latent_attention":
+                if m.get("rot") is None or int(m["rot"]["dims"]) != int(m["rot_dim"]):
+                    raise ConfigError(f"config.json: layer {i}: rot.dims must be rot_dim")
+                if int(m.get("q_rank", 0) or 0) < 0:
+                    raise ConfigError(f"config.json: layer {i}: q_rank must not be negative")
+            mlp = layer.get("mlp")
+            if mlp is None:
+                continue
+            if mlp.get("kind") == "dense":
+                if not int(mlp.get("ff", 0)) > 0:
+                    raise ConfigError(f"config.json: layer {i}: a dense mlp needs a positive ff")
+            elif mlp.get("kind") == "moe":
+                r = mlp.get("router") or {}
+                if not int((mlp.get("expert") or {}).get("ff", 0)) > 0 or not (0 < int(r.get("top", 0)) <= int(r.get("experts", 0))):
+                    raise ConfigError(f"config.json: layer {i}: a moe mlp needs expert.ff, router.experts and router.top "
+                                      "(at most the experts)")
+                if mlp.get("shared") is not None and not int(mlp["shared"].get("ff", 0)) > 0:
+                    raise ConfigError(f"config.json: layer {i}: a shared expert needs a positive ff")
+            else:
+                raise ConfigError(f"config.json: layer {i}: mlp.kind {mlp.get('kind')!r} is neither 'dense' nor 'moe'")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"architecture": self.architectures[0] if self.architectures else "Kegozen",
+             "layers": json.loads(json.dumps(list(self.layers))), "norm": {"eps": self.norm_eps},
+             "vocab": self.vocab_size, "width": self.hidden_size}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

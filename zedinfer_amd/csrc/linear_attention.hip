@@ -86,7 +86,7 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
                         const float* __restrict__ head_decay, float* __restrict__ state, int64_t state_stride,
                         const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                         const int32_t* __restrict__ entry_past, const int32_t* __restrict__ entry_slot, int heads,
-                        int dim, int vdim, int act, float qscale) {
+                        int dim, int vdim, int act, float qscale, int share, int decay_heads) {
     constexpr int D = LA_PARTS * R;               // rows the lanes of a column hold
     constexpr int DP = la_place(D);               // floats of a staged row
     constexpr int NSEG = GATED ? 3 : 2;           // k, q (, decay)
@@ -114,7 +114,8 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
         S[r] = (!fresh && row < dim) ? S_[(int64_t)row * vdim + colc] : 0.f;
     }
     const float hd = head_decay ? head_decay[head] : 1.f;
-    const int64_t qk_at = (int64_t)head * dim, v_at = (int64_t)head * vdim;
+    // `share` heads in a row read the same q and k; a decay of one number a (token, head) is staged for every row
+    const int64_t qk_at = (int64_t)(head / share) * dim, v_at = (int64_t)head * vdim;
 
     // global -> registers: the chunk of tokens from `base` on.  Every load is issued, from addresses clamped into
     // the entry; what a thread must not use is zeroed when it goes to LDS.
@@ -133,7 +134,9 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
             for (int u = 0; u < PSEG; ++u) {
                 const int idx = u * THREADS + tid, tt = idx / D, d = idx % D;
                 const bool ok = tt < n_in && d < dim;
-                pre[seg * PSEG + u] = src[(int64_t)(tb + (ok ? tt : 0)) * stride + qk_at + (ok ? d : 0)];
+                const int64_t at = seg == 2 ? (decay_heads ? (int64_t)head : (int64_t)head * dim + (ok ? d : 0))
+                                            : qk_at + (ok ? d : 0);
+                pre[seg * PSEG + u] = src[(int64_t)(tb + (ok ? tt : 0)) * stride + at];
                 ok_bits |= (unsigned)ok << (seg * PSEG + u);
             }
         }
@@ -225,21 +228,25 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
     }
 }
 
-// out [n][heads*vdim] float32 (row stride ldo).  q, k [n][heads*dim] and v [n][heads*vdim]: float32, one row stride
-// `ld` (columns of one projection).  decay [n][heads*dim] float32 (row stride ld_decay) or null; head_decay [heads]
-// or null (then 1).  state [slots][state_stride] float32, of which this layer's heads*dim*vdim floats start at the
-// pointer given.  act 1: SiLU of q, k and v as they are read.  q is multiplied by qscale.
-extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, const float* k, const float* v, int64_t ld,
-                                   const float* decay, int64_t ld_decay, const float* head_decay, float* state,
-                                   int64_t state_stride, const int32_t* entry_start, const int32_t* entry_len,
-                                   const int32_t* entry_past, const int32_t* entry_slot, int entries, int heads,
-                                   int dim, int vdim, int act, float qscale, hipStream_t stream) {
+// out [n][heads*vdim] float32 (row stride ldo).  q, k [n][(heads/share)*dim] and v [n][heads*vdim]: float32, one row
+// stride `ld` (columns of one projection); `share` heads in a row read the same q and k.  decay float32 (row stride
+// ld_decay): [n][heads*dim], or with `decay_heads` [n][heads], one factor a (token, head); or null; head_decay
+// [heads] or null (then 1).  state [slots][state_stride] float32, of which this layer's heads*dim*vdim floats start at
+// the pointer given.  act 1: SiLU of q, k and v as they are read.  q is multiplied by qscale.
+extern "C" int zi_linear_attention_grouped(float* out, int64_t ldo, const float* q, const float* k, const float* v,
+                                           int64_t ld, const float* decay, int64_t ld_decay, const float* head_decay,
+                                           float* state, int64_t state_stride, const int32_t* entry_start,
+                                           const int32_t* entry_len, const int32_t* entry_past,
+                                           const int32_t* entry_slot, int entries, int heads, int dim, int vdim, int act,
+                                           float qscale, int share, int decay_heads, hipStream_t stream) {
     ZI_REQUIRE(entries >= 0 && entries <= 65535 && heads > 0 && heads <= 65535 && dim > 0 && vdim > 0,
                "linear_attention: bad sizes");
+    ZI_REQUIRE(share > 0 && heads % share == 0, "linear_attention: %d heads do not share q and k in runs of %d", heads, share);
     ZI_REQUIRE(dim <= 512, "linear_attention: dim %d is more than the 512 rows a wavefront holds", dim);
     ZI_REQUIRE(state_stride >= (int64_t)heads * dim * vdim, "linear_attention: the state row is too short");
-    ZI_REQUIRE(ldo >= (int64_t)heads * vdim && ld >= (int64_t)heads * dim && ld >= (int64_t)heads * vdim &&
-               (!decay || ld_decay >= (int64_t)heads * dim), "linear_attention: row stride too small");
+    ZI_REQUIRE(ldo >= (int64_t)heads * vdim && ld >= (int64_t)(heads / share) * dim && ld >= (int64_t)heads * vdim &&
+               (!decay || ld_decay >= (int64_t)heads * (decay_heads ? 1 : dim)), "linear_attention: row stride too small");
+    ZI_REQUIRE(!decay_heads || decay, "linear_attention: a decay a head and token must be given");
     ZI_REQUIRE(act == 0 || act == 1, "linear_attention: unknown activation %d", act);
     if (entries == 0) return 0;
     const dim3 grid((vdim + LA_WCOLS - 1) / LA_WCOLS, heads, entries);
@@ -247,11 +254,11 @@ extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, cons
     if (decay)                                                                                                       \
         linear_attention_kernel<R, TC, true><<<grid, LA_WAVES * ZI_WAVE, 0, stream>>>(                               \
             out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride, entry_start, entry_len,         \
-            entry_past, entry_slot, heads, dim, vdim, act, qscale);                                                  \
+            entry_past, entry_slot, heads, dim, vdim, act, qscale, share, decay_heads);                              \
     else                                                                                                             \
         linear_attention_kernel<R, TC, false><<<grid, LA_WAVES * ZI_WAVE, 0, stream>>>(                              \
             out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride, entry_start, entry_len,         \
-            entry_past, entry_slot, heads, dim, vdim, act, qscale)
+            entry_past, entry_slot, heads, dim, vdim, act, qscale, share, decay_heads)
     if (dim <= 32) { ZI_LA(2, 16); }
     else if (dim <= 64) { ZI_LA(4, 16); }
     else if (dim <= 128) { ZI_LA(8, 16); }
@@ -259,6 +266,16 @@ extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, cons
     else { ZI_LA(32, 4); }
 #undef ZI_LA
     return zi_check_launch("linear_attention");
+}
+
+extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, const float* k, const float* v, int64_t ld,
+                                   const float* decay, int64_t ld_decay, const float* head_decay, float* state,
+                                   int64_t state_stride, const int32_t* entry_start, const int32_t* entry_len,
+                                   const int32_t* entry_past, const int32_t* entry_slot, int entries, int heads,
+                                   int dim, int vdim, int act, float qscale, hipStream_t stream) {
+    return zi_linear_attention_grouped(out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride,
+                                       entry_start, entry_len, entry_past, entry_slot, entries, heads, dim, vdim, act,
+                                       qscale, 1, 0, stream);
 }
 
 #define GATE_SIGMOID 0

@@ -431,3 +431,121 @@ extern "C" int zi_moe_combine(float* out, const float* y, const float* wt, const
     moe_combine_kernel<<<n, 256, 0, stream>>>(out, y, wt, place_of, top, hidden);
     return zi_check_launch("moe_combine");
 }
+
+// ---- a router of independent scores --------------------------------------------------------------------------
+// s = sigmoid(z); the `top` experts with the largest s are chosen (the lowest index among equals); their weights are
+// the scores themselves, not renormalised.  z [n][ld] float32 of which the first E columns are the experts'.
+template <int PER>
+__global__ void __launch_bounds__(256)
+moe_route_sigmoid_kernel(int32_t* __restrict__ idx, float* __restrict__ wt, const float* __restrict__ z, int64_t ld,
+                         int n, int E, int top) {
+    const int lane = threadIdx.x % ZI_WAVE;
+    const int t = blockIdx.x * (blockDim.x / ZI_WAVE) + threadIdx.x / ZI_WAVE;
+    if (t >= n) return;
+    float choice[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = lane + i * ZI_WAVE;
+        choice[i] = e < E ? 1.f / (1.f + expf(-z[(int64_t)t * ld + e])) : -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + i * ZI_WAVE;
+            if (e < E && (choice[i] > best || (choice[i] == best && e < best_e))) {
+                best = choice[i];
+                best_e = e;
+            }
+        }
+#pragma unroll
+        for (int o = ZI_WAVE / 2; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, ZI_WAVE);
+            const int oe = __shfl_xor(best_e, o, ZI_WAVE);
+            if (ob > best || (ob == best && oe < best_e)) {
+                best = ob;
+                best_e = oe;
+            }
+        }
+        if (lane == 0) {
+            idx[(int64_t)t * top + k] = best_e;
+            wt[(int64_t)t * top + k] = best;
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (lane + i * ZI_WAVE == best_e) choice[i] = -INFINITY;
+    }
+}
+
+extern "C" int zi_moe_route_sigmoid(int32_t* idx, float* wt, const float* z, int64_t ld, int n, int experts, int top,
+                                    hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && experts > 0 && experts <= MOE_MAX_EXPERTS && top > 0 && top <= experts && ld >= experts,
+               "moe_route_sigmoid: bad sizes (experts %d, top %d; at most %d experts)", experts, top, MOE_MAX_EXPERTS);
+    if (n == 0) return 0;
+    const int blocks = (n + 3) / 4;
+#define ZI_MOE_ROUTE(PER) moe_route_sigmoid_kernel<PER><<<blocks, 256, 0, stream>>>(idx, wt, z, ld, n, experts, top)
+    if (experts <= ZI_WAVE) ZI_MOE_ROUTE(1);
+    else if (experts <= 2 * ZI_WAVE) ZI_MOE_ROUTE(2);
+    else if (experts <= 4 * ZI_WAVE) ZI_MOE_ROUTE(4);
+    else ZI_MOE_ROUTE(MOE_PER_LANE);
+#undef ZI_MOE_ROUTE
+    return zi_check_launch("moe_route_sigmoid");
+}
+
+// The gated middle of experts whose INPUT carries the routing weight: an expert is linear up to its activation, so
+// gate (w x) = w gate(x) and up (w x) = w up(x): out = silu(w g) * (w u) for row r of the grouped pairs, w the weight
+// of the pair that stands at place r (wt[order[r]]).  gu [pairs][2 ff] float32 (gate, then up).
+template <typename TO>
+__global__ void __launch_bounds__(256)
+moe_weighted_glu_kernel(TO* __restrict__ out, int64_t ldo, const float* __restrict__ gu, int64_t ld,
+                        const float* __restrict__ wt, const int32_t* __restrict__ order, int pairs, int ff) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)pairs * ff) return;
+    const int64_t r = i / ff, c = i % ff;
+    const float w = wt[order[r]];
+    const float g = w * gu[r * ld + c], u = w * gu[r * ld + ff + c];
+    zi_store(out + r * ldo + c, g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int zi_moe_weighted_glu(void* out, int out_dt, int64_t ldo, const float* gu, int64_t ld, const float* wt,
+                                   const int32_t* order, int pairs, int ff, hipStream_t stream) {
+    ZI_REQUIRE(pairs >= 0 && ff > 0 && ld >= 2 * (int64_t)ff && ldo >= ff, "moe_weighted_glu: bad sizes");
+    if (pairs == 0) return 0;
+    const int64_t total = (int64_t)pairs * ff;
+    ZI_DISPATCH_DTYPE(out_dt, TO, {
+        moe_weighted_glu_kernel<TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>((TO*)out, ldo, gu, ld, wt, order,
+                                                                                         pairs, ff);
+    });
+    return zi_check_launch("moe_weighted_glu");
+}
+
+// out [n][H] = sum over a token's `top` pairs of y[place_of[pair]] (each counts once: the weight went into the
+// expert's input) + sigmoid(gate[t * ld_gate]) * shared[t], where shared is the sum of `splits` float32 terms
+// (`split_stride` apart) or null.
+__global__ void __launch_bounds__(256)
+moe_sum_shared_kernel(float* __restrict__ out, const float* __restrict__ y, const int32_t* __restrict__ place_of,
+                      const float* __restrict__ shared, int splits, int64_t split_stride, const float* __restrict__ gate,
+                      int64_t ld_gate, int top, int H) {
+    const int64_t t = blockIdx.x;
+    const float gs = (shared && gate) ? 1.f / (1.f + expf(-gate[t * ld_gate])) : 1.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) acc += y[(int64_t)place_of[t * top + k] * H + c];
+        if (shared) {
+            float sv = shared[t * H + c];
+            for (int s = 1; s < splits; ++s) sv += shared[s * split_stride + t * H + c];
+            acc += gs * sv;
+        }
+        out[t * H + c] = acc;
+    }
+}
+
+extern "C" int zi_moe_sum_shared(float* out, const float* y, const int32_t* place_of, const float* shared, int splits,
+                                 int64_t split_stride, const float* gate, int64_t ld_gate, int n, int top, int hidden,
+                                 hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && top > 0 && hidden > 0 && splits >= 1, "moe_sum_shared: bad sizes");
+    if (n == 0) return 0;
+    moe_sum_shared_kernel<<<n, 256, 0, stream>>>(out, y, place_of, shared, splits, split_stride, gate, ld_gate, top, hidden);
+    return zi_check_launch("moe_sum_shared");
+}

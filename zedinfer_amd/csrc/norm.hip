@@ -216,3 +216,65 @@ extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* d
     })));
     return zi_check_launch("add_rmsnorm");
 }
+
+// ---- a norm on a sublayer's output, and the next sublayer's norm, in one pass over the row ------------------------
+// resid (float32, in place) += y / sqrt(mean(y^2) + eps) * w1, where y is the sum of `splits` terms (rising order)
+// and w1 the first gain (1 + w1 with add_one); then, when `out` is given, out = resid / sqrt(mean(resid^2) + eps2) *
+// w2 (1 + w2 with add_one): the norm that the next sublayer reads.  One workgroup a row; the row lies in LDS between
+// the passes.  The sums of squares are added in an order fixed by the row's width alone.
+template <typename TD, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+normed_add_norm_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD* __restrict__ y, int64_t ldy, int splits,
+                       int64_t split_stride, const TW* __restrict__ w1, const TW* __restrict__ w2, int H, float eps,
+                       float eps2, int add_one) {
+    extern __shared__ float row_values[];
+    __shared__ float scratch[16];
+    const int64_t t = blockIdx.x;
+    const TD* yr = y + t * ldy;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = zi_load(yr + i);
+        for (int s = 1; s < splits; ++s) v += zi_load(yr + s * split_stride + i);
+        row_values[i] = v;
+        ss += v * v;
+    }
+    ss = zi_block_sum(ss, scratch);
+    const float r = 1.f / sqrtf(ss / (float)H + eps);
+    float* rr = resid + t * H;
+    float ss2 = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float g = zi_load(w1 + i) + (add_one ? 1.f : 0.f);
+        const float v = rr[i] + row_values[i] * r * g;
+        rr[i] = v;
+        row_values[i] = v;
+        ss2 += v * v;
+    }
+    if (!out) return;
+    ss2 = zi_block_sum(ss2, scratch);
+    const float r2 = 1.f / sqrtf(ss2 / (float)H + eps2);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float g = zi_load(w2 + i) + (add_one ? 1.f : 0.f);
+        zi_store(out + t * H + i, row_values[i] * r2 * g);
+    }
+}
+
+// y: [n][hidden] rows of type y_dt (row stride ldy), or `splits` float32 terms `split_stride` apart; w1, w2 [hidden] of
+// type w_dt; out [n][hidden] of type out_dt, or null (then w2 is not read).
+extern "C" int zi_normed_add_norm(void* out, int out_dt, float* resid, const void* y, int y_dt, int64_t ldy, int splits,
+                                  int64_t split_stride, const void* w1, const void* w2, int w_dt, int n, int hidden,
+                                  float eps, float eps2, int add_one, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && hidden > 0 && hidden <= 15360 && ldy >= hidden && splits >= 1 && eps > 0.f && (!out || (w2 && eps2 > 0.f)),
+               "normed_add_norm: bad sizes (hidden %d)", hidden);
+    ZI_REQUIRE(splits == 1 || y_dt == ZI_F32, "normed_add_norm: partial sums are float32");
+    if (n == 0) return 0;
+    const size_t lds = (size_t)hidden * sizeof(float);
+    ZI_DISPATCH_DTYPE(y_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, {
+        if (!out || out_dt == ZI_F32)
+            normed_add_norm_kernel<TD, TW, float><<<n, 256, lds, stream>>>((float*)out, resid, (const TD*)y, ldy, splits,
+                split_stride, (const TW*)w1, (const TW*)w2, hidden, eps, eps2, add_one);
+        else
+            normed_add_norm_kernel<TD, TW, zi_bf16><<<n, 256, lds, stream>>>((zi_bf16*)out, resid, (const TD*)y, ldy, splits,
+                split_stride, (const TW*)w1, (const TW*)w2, hidden, eps, eps2, add_one);
+    }));
+    return zi_check_launch("normed_add_norm");
+}

@@ -249,6 +249,51 @@ int zi_attention_decode_biased(void* out, const void* q, int dt, int n_idx, int6
 // moe.hip
 int zi_moe_route_table(int32_t* idx, float* wt, const int32_t* ids, const int32_t* table, int n, int vocab, int
     experts, int top, hipStream_t stream);
+// rope_kv.hip
+int zi_rope_table_scaled(float* out, const int32_t* pos, const float* inv_freq, int n, int half, float magnitude,
+    hipStream_t stream);
+// linear_attention.hip
+int zi_linear_attention_grouped(float* out, int64_t ldo, const float* q, const float* k, const float* v, int64_t ld,
+    const float* decay, int64_t ld_decay, const float* head_decay, float* state, int64_t state_stride, const int32_t*
+    entry_start, const int32_t* entry_len, const int32_t* entry_past, const int32_t* entry_slot, int entries, int
+    heads, int dim, int vdim, int act, float qscale, int share, int decay_heads, hipStream_t stream);
+// ssm.hip
+int zi_ssm_prepare(float* out, int64_t ldo, const float* proj, int64_t ld, int n, const float* conv_w, const float*
+    conv_b, const float* dt_bias, const float* a_log, const float* state, int64_t state_stride, const int32_t*
+    tok_seq, const int32_t* entry_start, const int32_t* entry_slot, int heads, int vdim, int gn2, int taps,
+    hipStream_t stream);
+// ssm.hip
+int zi_ssm_finish(void* out, int out_dt, int64_t ldo, const float* y, int64_t ldy, const float* x, int64_t ldx, const
+    float* z, int64_t ldz, const float* skip, const float* gain, int n, int heads, int vdim, int parts, float eps,
+    hipStream_t stream);
+// pooled_attention.hip
+int zi_norm_rope_store(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const float* proj, int64_t ld,
+    int splits, int64_t split_stride, const float* q_gain, const float* k_gain, float eps, const float* table, int rot,
+    const float* vtable, const int32_t* slots, int64_t cache_slots, int n, int nh, int nkv, int dim, int vdim,
+    hipStream_t stream);
+// pooled_attention.hip
+int zi_pool_blocks(float* kpool, float* vpool, int64_t pool_rows, const void* kcache, const void* vcache, int dt, const
+    int32_t* pool_slots, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables, int max_pages,
+    int num_pages, int page_size, int n, int nkv, int dim, int vdim, int pool, hipStream_t stream);
+// pooled_attention.hip
+int zi_pooled_attention(void* out, int64_t ldo, const void* q, int64_t ldq, int dt, const void* kcache, const void*
+    vcache, const float* kpool, const float* vpool, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int page_size, const int32_t* pool_tables, int pool_max_pages, int
+    pool_num_pages, int pool_page_size, int n, int nh, int nkv, int dim, int vdim, int window, int pool, float scale,
+    const float* vtable, hipStream_t stream);
+// norm.hip
+int zi_normed_add_norm(void* out, int out_dt, float* resid, const void* y, int y_dt, int64_t ldy, int splits, int64_t
+    split_stride, const void* w1, const void* w2, int w_dt, int n, int hidden, float eps, float eps2, int add_one,
+    hipStream_t stream);
+// moe.hip
+int zi_moe_route_sigmoid(int32_t* idx, float* wt, const float* z, int64_t ld, int n, int experts, int top,
+    hipStream_t stream);
+// moe.hip
+int zi_moe_weighted_glu(void* out, int out_dt, int64_t ldo, const float* gu, int64_t ld, const float* wt, const
+    int32_t* order, int pairs, int ff, hipStream_t stream);
+// moe.hip
+int zi_moe_sum_shared(float* out, const float* y, const int32_t* place_of, const float* shared, int splits, int64_t
+    split_stride, const float* gate, int64_t ld_gate, int n, int top, int hidden, hipStream_t stream);
 // sampling.hip
 int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int rows, int vocab, const float*
     temperature, const int32_t* top_k, const float* top_p, const float* penalty, const float* uniform, const int32_t*
@@ -319,5 +364,16 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_attention_prefill_biased) \
     X(zi_attention_decode_biased) \
     X(zi_moe_route_table) \
+    X(zi_rope_table_scaled) \
+    X(zi_linear_attention_grouped) \
+    X(zi_ssm_prepare) \
+    X(zi_ssm_finish) \
+    X(zi_norm_rope_store) \
+    X(zi_pool_blocks) \
+    X(zi_pooled_attention) \
+    X(zi_normed_add_norm) \
+    X(zi_moe_route_sigmoid) \
+    X(zi_moe_weighted_glu) \
+    X(zi_moe_sum_shared) \
     X(zi_argmax) \
     X(zi_sample)

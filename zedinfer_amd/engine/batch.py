@@ -279,6 +279,7 @@ class DecodeImage:
         self.image = np.empty(max(self.total, 1), dtype=np.int32)
         self.image[:self.total] = self.batch.host_image
         self.page_sizes = [g.page_size for g in cache.groups]
+        self.strides = [getattr(g, "stride", 1) for g in cache.groups]
         self.entries_made = E
         self.rows = np.arange(self.real)
 
@@ -315,7 +316,15 @@ class DecodeImage:
                         raise ValueError(f"block tables of group {g} need {len(pg)} columns, {w} given")
                     table[i, :len(pg)] = pg
                     table[i, len(pg):] = -1
-            ps = self.page_sizes[g]
+            ps, stride = self.page_sizes[g], self.strides[g]
+            if stride > 1:      # one row for every `stride` positions: a slot only where a position completes one
+                ends = (pos + 1) % stride == 0
+                row = pos // stride
+                pages = table[self.rows, np.minimum(row // ps, w - 1)]
+                if (pages[ends] < 0).any():
+                    raise RuntimeError("a decoded token's block has no page")
+                self.piece(FIXED_PIECES + 2 * g)[:E] = np.where(ends, pages * ps + row % ps, -1)
+                continue
             pages = table[self.rows, pos // ps]
             if (pages < 0).any():
                 raise RuntimeError("a decoded token's position has no page")

@@ -1,4 +1,4 @@
-from . import dedelorn, qwen2, tilivik, tosisun  # noqa: F401  (register the architectures)
+from . import dedelorn, kegozen, qwen2, tilivik, tosisun  # noqa: F401  (register the architectures)
 from .model import DecoderModel, expected_weights
 
-__all__ = ["DecoderModel", "expected_weights", "dedelorn", "qwen2", "tilivik", "tosisun"]
+__all__ = ["DecoderModel", "expected_weights", "dedelorn", "kegozen", "qwen2", "tilivik", "tosisun"]

@@ -114,6 +114,11 @@ class DecoderModel:
                     out[st.cache] = KVCacheRequest("full", 0, req.tensors)
                 else:
                     out[st.cache] = KVCacheRequest(req.kind, max(had.window, req.window), req.tensors)
+        # a mixer's further caches, under (cache id, name), for the runs that write
+        for st in self.fc.schedule:
+            if st.writes_cache:
+                for name, req in self.blocks[st.layer].mixer.side_cache_requests().items():
+                    out[(st.cache, name)] = req
         return out
 
     def state_requests(self) -> Dict[int, StateRequest]:

@@ -27,6 +27,10 @@ from .sublayers import (clamped_glu, conv_qkv, conv_state_floats, conv_tail, con
 from .recurrent import (attention_biased, embedding_sum, gate_heads, gated_rms_norm_act, linear_attention,
                         linear_attention_state_floats, lowrank_decay, moe_route_table, normed_kv_store, stream_reenter,
                         token_shift)
+from . import hybrid
+from .hybrid import (linear_attention_grouped, moe_route_sigmoid, moe_sum_shared, moe_weighted_glu, norm_rope_store,
+                     normed_add_norm, pool_blocks, pooled_attention, rope_table_scaled, ssm_finish, ssm_prepare,
+                     ssm_state_floats)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
@@ -48,5 +52,7 @@ __all__ = [
     "softcap",
     "attention_biased", "embedding_sum", "gate_heads", "gated_rms_norm_act", "linear_attention",
     "linear_attention_state_floats", "lowrank_decay", "moe_route_table", "normed_kv_store", "stream_reenter", "token_shift",
+    "linear_attention_grouped", "moe_route_sigmoid", "moe_sum_shared", "moe_weighted_glu", "norm_rope_store",
+    "normed_add_norm", "pool_blocks", "pooled_attention", "rope_table_scaled", "ssm_finish", "ssm_prepare", "ssm_state_floats",
     "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

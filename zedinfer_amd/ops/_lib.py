@@ -111,6 +111,17 @@ _PROTOTYPES = {
                                     P, F, P, I, I, P],
     "zi_attention_decode_biased": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P, F, P, I, I, P],
     "zi_moe_route_table": [P, P, P, P, I, I, I, I, P],
+    "zi_rope_table_scaled": [P, P, P, I, I, F, P],
+    "zi_linear_attention_grouped": [P, L, P, P, P, L, P, L, P, P, L, P, P, P, P, I, I, I, I, I, F, I, I, P],
+    "zi_ssm_prepare": [P, L, P, L, I, P, P, P, P, P, L, P, P, P, I, I, I, I, P],
+    "zi_ssm_finish": [P, I, L, P, L, P, L, P, L, P, P, I, I, I, I, F, P],
+    "zi_norm_rope_store": [P, I, L, P, P, P, L, I, L, P, P, F, P, I, P, P, L, I, I, I, I, I, P],
+    "zi_pool_blocks": [P, P, L, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
+    "zi_pooled_attention": [P, L, P, L, I, P, P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, I, F, P, P],
+    "zi_normed_add_norm": [P, I, P, P, I, L, I, L, P, P, I, I, I, F, F, I, P],
+    "zi_moe_route_sigmoid": [P, P, P, L, I, I, I, P],
+    "zi_moe_weighted_glu": [P, I, L, P, L, P, P, I, I, P],
+    "zi_moe_sum_shared": [P, P, P, P, I, L, P, L, I, I, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
     "zi_tape_record_many": [P, c_char_p, P, P, I],
     "zi_tape_run": [P, P],

@@ -160,12 +160,18 @@ class KVCacheRequest:
     positions ("window"; with ``keep_first`` the pages of a sequence's first ``keep_first`` positions are kept as
     well when the window has passed them), and in every page the named ``tensors`` (name, PageTensor).  The cache manager
     allocates [pages, *page shape] for each and hands them to the mixer's runs by name
-    (``LayerMemory.tensors``); what they hold and how they are laid out is the mixer's business."""
+    (``LayerMemory.tensors``); what they hold and how they are laid out is the mixer's business.
+
+    ``stride`` > 1 (with kind "full"): the cache holds one row for every ``stride`` positions, not one a position: row
+    b belongs to the positions b * stride .. b * stride + stride - 1 and is written when the last of them arrives (a
+    summary of a block of positions).  A page then spans ``page_size * stride`` positions, and a token's slot in such a
+    cache is the row its position completes, or -1 when it completes none."""
 
     kind: str
     window: int = 0
     tensors: Tuple[Tuple[str, PageTensor], ...] = ()
     keep_first: int = 0
+    stride: int = 1
 
 
 @dataclass(frozen=True)
@@ -184,6 +190,9 @@ class LayerMemory:
     tensors: Dict[str, torch.Tensor] = field(default_factory=dict)   # name -> [pages, *page shape], as requested
     writes: bool = True
     state: Optional[torch.Tensor] = None  # [slots, *StateRequest.shape]
+    # what the mixer's further caches (``Mixer.side_cache_requests``) were bound to, by their names; each has a group
+    # and tensors of its own
+    sides: Dict[str, "LayerMemory"] = field(default_factory=dict)
 
 
 class Part:
@@ -309,6 +318,12 @@ class Mixer(Part):
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return None
+
+    def side_cache_requests(self) -> Dict[str, KVCacheRequest]:
+        """Further paged caches beside the one of ``cache_request``, by a name of the mixer's choice: each is kept in
+        a group that fits its kind (one row a position over all positions or a window, or one row for every so many
+        positions) and comes back as ``memory.sides[name]`` (its ``group`` indexes ``batch.groups``)."""
+        return {}
 
     def state_request(self) -> Optional[StateRequest]:
         return None

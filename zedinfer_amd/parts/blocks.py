@@ -130,3 +130,37 @@ class OutputNormBlock(Block):
         if shared is not None:
             shared[self.SHARED] = x
         return None
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """h += norm_mixer_out(mixer(norm_in(h))); h += norm_ff_out(feed_forward(norm_ff_in(h))): a norm before and a
+    norm after each sublayer.  The norms on the outputs must offer ``add_normed`` (the RMS norm does): the output's
+    norm, the addition into the float32 stream and the norm that the feed-forward reads are one launch.  Nothing is
+    left pending: the stream is whole when the block returns.  The feed-forward may be the kind "none" (its two
+    norms are then the kind "none" too)."""
+
+    graph_safe = True
+    tape_safe = True
+
+    norm_names = ("input", "mixer_out", "ff_in", "ff_out")
+
+    def __init__(self, norms, mixer, feed_forward, rt: Runtime):
+        self.norm_in, self.norm_mixer_out = norms["input"], norms["mixer_out"]
+        self.norm_ff_in, self.norm_ff_out = norms["ff_in"], norms["ff_out"]
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.has_ff = getattr(feed_forward, "kind", "") != "none"
+        self.rt = rt
+
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, memory: LayerMemory):
+        x = self.norm_in.add_forward(resid, delta) if delta is not None else self.norm_in.forward(resid)
+        a = self.mixer.forward(x, batch, memory)
+        if not self.has_ff:
+            self.norm_mixer_out.add_normed(resid, a)
+            return None
+        y = self.norm_mixer_out.add_normed(resid, a, then=self.norm_ff_in)
+        kw = {"batch": batch} if self.feed_forward.reads_batch else {}
+        f = self.feed_forward.forward(y, **kw)
+        self.norm_ff_out.add_normed(resid, f)
+        return None

@@ -521,3 +521,95 @@ class TableExperts(FeedForward):
         if out is None:
             out = rt.buffer("moe_out", (n, self.hidden), torch.float32)
         return ops.moe_combine(y, wt, place_of, out)
+
+
+@register_feed_forward("scored_experts")
+class ScoredExperts(FeedForward):
+    """A mixture of small gated feed-forwards down_e(silu(gate_e h) * up_e h), no biases, of which every token uses
+    ``top``, plus, optionally, a shared one that every token uses.
+
+    Router: z = W_router x in float32, s = sigmoid(z): every expert is scored by itself.  The ``top`` experts with the
+    largest scores are chosen (the lowest index among equals); their weights are the scores, not renormalised.  The
+    weight multiplies the expert's INPUT: the result is the sum of expert_e(s_e x) over the chosen experts.  An
+    expert is linear before its activation, so the kernels compute silu(s g) * (s u) from g = gate_e x and u = up_e x
+    (``ops.moe_weighted_glu``) instead of scaling rows of x.  The shared expert's output is multiplied by
+    sigmoid(w_sg . x), one number a token (``shared_gate``); its row is stacked under the router's, one product.
+
+    Routing, grouping and the experts' products run on the device as for the other mixtures (``csrc/moe.hip``): the
+    launches of a step do not depend on what the tokens choose.  The result is float32 [n, hidden].
+    params: hidden_size, experts, top, ff, shared_ff (0: none), shared_gate (whether the shared expert is gated)."""
+
+    graph_safe = True
+    tape_safe = True
+    writes_into = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, E, ff, sff = int(p["hidden_size"]), int(p["experts"]), int(p["ff"]), int(p.get("shared_ff", 0) or 0)
+        w = {"router": WeightSpec((E, H))}
+        for e in range(E):
+            w[f"gate_{e}"] = WeightSpec((ff, H))
+            w[f"up_{e}"] = WeightSpec((ff, H))
+            w[f"down_{e}"] = WeightSpec((H, ff))
+        if sff:
+            w.update({"shared_gate": WeightSpec((sff, H)), "shared_up": WeightSpec((sff, H)),
+                      "shared_down": WeightSpec((H, sff))})
+            if p.get("shared_gate", False):
+                w["shared_sg"] = WeightSpec((1, H))
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.experts, self.top, self.ff = int(p["hidden_size"]), int(p["experts"]), int(p["top"]), int(p["ff"])
+        if not (0 < self.top <= self.experts):
+            raise ValueError(f"scored_experts: top {self.top} of {self.experts} experts")
+        E = self.experts
+        self.sff = int(p.get("shared_ff", 0) or 0)
+        self.gated_shared = bool(self.sff and p.get("shared_gate", False))
+        # the router's rows, then the shared expert's gate row, padded to a multiple of 8 rows: one product
+        rows = E + (1 if self.gated_shared else 0)
+        r = weights["router"]
+        stacked = torch.zeros((-(-rows // 8) * 8, self.hidden), dtype=r.dtype, device=r.device)
+        stacked[:E] = r
+        if self.gated_shared:
+            stacked[E] = weights["shared_sg"].reshape(-1).to(r.dtype)
+        self.router = stacked
+        self.gate_up = torch.stack([torch.cat([weights[f"gate_{e}"], weights[f"up_{e}"].to(weights[f"gate_{e}"].dtype)])
+                                    for e in range(E)]).contiguous()
+        self.down = torch.stack([weights[f"down_{e}"] for e in range(E)]).contiguous()
+        self.shared = None
+        if self.sff:
+            self.shared = GatedMLP(PartSpec("gated_mlp", {"hidden_size": self.hidden, "intermediate_size": self.sff,
+                                                          "activation": "silu"}),
+                                   {"gate": weights["shared_gate"], "up": weights["shared_up"], "down": weights["shared_down"]}, rt)
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        n, E, top, ff, rt = x.shape[0], self.experts, self.top, self.ff, self.rt
+        pairs = n * top
+        z = ops.linear(x, self.router, out=rt.buffer("moe_logits", (n, self.router.shape[0]), torch.float32))
+        idx = rt.buffer("moe_choice", (n, top), torch.int32)
+        wt = rt.buffer("moe_weight", (n, top), torch.float32)
+        ops.moe_route_sigmoid(z, E, top, idx, wt)
+        rows = ops.moe_tile_rows(x.dtype, self.gate_up.dtype, (self.hidden, ff), pairs, E)
+        tiles = ops.moe_max_tiles(pairs, E, rows)
+        plan = rt.buffer("moe_plan", (1 + 3 * tiles,), torch.int32)
+        order = rt.buffer("moe_order", (pairs,), torch.int32)
+        place_of = rt.buffer("moe_place", (pairs,), torch.int32)
+        ops.moe_group(idx, E, rows, plan, order, place_of)
+        gu = rt.buffer("moe_gate_up", (pairs, 2 * ff), torch.float32)
+        ops.moe_linear(x, self.gate_up, plan, rows, tiles, out=gu, source=order, source_div=top)
+        act = rt.buffer("moe_act", (pairs, ff))
+        ops.moe_weighted_glu(gu, wt, order, ff, out=act)
+        y = rt.buffer("moe_out_rows", (pairs, self.hidden), torch.float32)
+        ops.moe_linear(act, self.down, plan, rows, tiles, out=y)
+        shared = None
+        if self.shared is not None:
+            shared = self.shared.forward(x, out=rt.buffer("moe_shared_out", (n, self.hidden), torch.float32))
+        if out is None:
+            out = rt.buffer("moe_out", (n, self.hidden), torch.float32)
+        return ops.moe_sum_shared(y, place_of, top, out, shared=shared, gate=z[:, E] if self.gated_shared else None)

@@ -34,8 +34,15 @@ class LatentAttention(Mixer):
     A layer built with ``shares_cache`` has no W_dkv: its run of the schedule names the cache of the layer whose
     latents it reads (``ScheduleStep.writes_cache`` False), and it brings its own W_uk, W_uv, queries, window.
 
-    params: hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, window (0: all keys), eps, shares_cache,
-    position (a PartSpec of an encoding that hands over ``pair_table``: neighbouring pairs turn)."""
+    With ``q_rank`` the queries come through a latent of their own: c_q = rms_norm(W_dq x) * g_q, q = W_uq c_q
+    (two products and a norm instead of the one product W_q x).
+
+    ``pairing`` says which of the rot_dim dims a checkpoint pairs: "interleaved" (2i with 2i + 1, what the kernels
+    turn; the default) or "halves" (i with i + rot_dim / 2: the turned rows of the query and key projections are
+    reordered at load, the same way in both, which changes no score).
+
+    params: hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, window (0: all keys), eps, shares_cache, q_rank
+    (0: none), pairing, position (a PartSpec of an encoding that hands over ``pair_table``: neighbouring pairs turn)."""
 
     graph_safe = True
     tape_safe = True
@@ -46,8 +53,13 @@ class LatentAttention(Mixer):
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         p = spec.params
         H, nh, dim, rot, vdim, rank = (int(p[k]) for k in ("hidden_size", "heads", "dim", "rot_dim", "vdim", "kv_rank"))
-        w = {"q": WeightSpec((nh * (dim + rot), H)), "uk": WeightSpec((nh * dim, rank)),
-             "uv": WeightSpec((nh * vdim, rank)), "o": WeightSpec((H, nh * vdim))}
+        w = {"uk": WeightSpec((nh * dim, rank)), "uv": WeightSpec((nh * vdim, rank)), "o": WeightSpec((H, nh * vdim))}
+        q_rank = int(p.get("q_rank", 0) or 0)
+        if q_rank:
+            w.update({"dq": WeightSpec((q_rank, H)), "dq_norm": WeightSpec((q_rank,), init="ones"),
+                      "uq": WeightSpec((nh * (dim + rot), q_rank))})
+        else:
+            w["q"] = WeightSpec((nh * (dim + rot), H))
         if not p.get("shares_cache", False):
             w["dkv"] = WeightSpec((rank + rot, H))
             w["dkv_norm"] = WeightSpec((rank,), init="ones")
@@ -68,7 +80,24 @@ class LatentAttention(Mixer):
         self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, {}, rt)
         if self.rot and (not hasattr(self.position, "pair_table") or self.position.rotary_dim != self.rot):
             raise ValueError("latent_attention: the position encoding must turn neighbouring pairs of all rot_dim dims")
-        self.q, self.uk, self.uv, self.o = weights["q"], weights["uk"], weights["uv"], weights["o"]
+        self.uk, self.uv, self.o = weights["uk"], weights["uv"], weights["o"]
+        self.q_rank = int(p.get("q_rank", 0) or 0)
+        pairing = str(p.get("pairing", "interleaved"))
+        if pairing not in ("interleaved", "halves"):
+            raise ValueError(f"latent_attention: unknown pairing {pairing!r}")
+        # pairs (i, i + rot/2) of a checkpoint become the neighbours (2i, 2i + 1) that the kernels turn
+        order = None
+        if pairing == "halves" and self.rot:
+            half = self.rot // 2
+            order = torch.tensor([j // 2 + (j % 2) * half for j in range(self.rot)], dtype=torch.long, device=self.uk.device)
+        q_w = weights["uq"] if self.q_rank else weights["q"]
+        if order is not None:
+            per_head = q_w.view(self.nh, self.dim + self.rot, q_w.shape[1]).clone()
+            per_head[:, self.dim:] = per_head[:, self.dim:][:, order]
+            q_w = per_head.reshape(self.nh * (self.dim + self.rot), q_w.shape[1]).contiguous()
+        self.q = q_w
+        if self.q_rank:
+            self.dq, self.dq_norm = weights["dq"], weights["dq_norm"]
         # a bfloat16 cache of sizes the matrix-core kernel takes goes there; everything else to the plain kernel
         self.cores = (rt.device.type == "cuda" and rt.dtype == torch.bfloat16
                       and ops.latent_attention_cores_supported(rt.dtype, self.rank, self.rot))
@@ -79,6 +108,8 @@ class LatentAttention(Mixer):
             self.uk_t = self.uk.view(self.nh, self.dim, self.rank).transpose(1, 2).contiguous()
         if not self.shares_cache:
             self.dkv = weights["dkv"]
+            if order is not None:
+                self.dkv = torch.cat([self.dkv[:self.rank], self.dkv[self.rank:][order]]).contiguous()
             self.dkv_norm = weights["dkv_norm"]
 
     def cache_request(self) -> Optional[KVCacheRequest]:
@@ -97,6 +128,9 @@ class LatentAttention(Mixer):
                 raise ValueError("latent_attention: a layer without W_dkv cannot write a cache")
             dkv = ops.linear(x, self.dkv, out=rt.buffer("latent_dkv", (n, self.rank + self.rot), torch.float32))
             ops.latent_store(dkv, self.dkv_norm, self.eps, table, view.slots, c_cache, kr_cache, self.rank, self.rot)
+        if self.q_rank:
+            cq = ops.linear(x, self.dq, out=rt.buffer("latent_cq", (n, self.q_rank), torch.float32))
+            x = ops.rms_norm(cq, self.dq_norm, self.eps, out=rt.buffer("latent_cq_normed", (n, self.q_rank)))
         q = ops.linear(x, self.q, out=rt.buffer("latent_q", (n, self.nh * (self.dim + self.rot)), torch.float32))
         qa = rt.buffer("latent_qa", (n, self.nh, self.rank + self.rot), torch.float32)
         ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa, w_uk_t=self.uk_t)

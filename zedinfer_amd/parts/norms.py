@@ -48,6 +48,19 @@ class RMSNorm(Norm):
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out=out, add_one=self.add_one)
 
 
+    def add_normed(self, resid: torch.Tensor, y: torch.Tensor, then: Optional["RMSNorm"] = None) -> Optional[torch.Tensor]:
+        """The norm on a sublayer's OUTPUT: resid (float32, in place) += norm(y); y is [n, dim] or a stack [S, n, dim]
+        of float32 terms that are added first.  With ``then`` (the norm the next sublayer reads, of this norm's kind)
+        the new rows of the stream come back normed by it, from the same launch."""
+        out = None
+        if then is not None:
+            if then.add_one != self.add_one or then.weight.dtype != self.weight.dtype:
+                raise ValueError("rmsnorm: the two norms of one launch must be of one kind")
+            out = self.rt.buffer("norm_out", (resid.shape[0], self.dim), then.out_dtype or self.rt.dtype)
+        return ops.normed_add_norm(resid, y, self.weight, self.eps, self.add_one, w2=then.weight if then is not None else None,
+                                   eps2=then.eps if then is not None else 0.0, out=out)
+
+
 @register_norm("none")
 class NoNorm(Norm):
     """Stands where a block arrangement names a norm that a layer does not have (the norm before a feed-forward
