@@ -159,8 +159,9 @@ def attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m, eps: float, round_
     q = (h @ w["q"].T).reshape(T, H, d)
     k = (h @ w["k"].T).reshape(T, G, d)
     v = (h @ w["v"].T).reshape(T, G, vd)
-    q = rms(q, eps) * w["q.norm"]
-    k = rms(k, eps) * w["k.norm"]
+    if "q.norm" in w:
+        q = rms(q, eps) * w["q.norm"]
+        k = rms(k, eps) * w["k.norm"]
     rot = m.get("rot")
     pos = list(range(T))
     if rot:
@@ -185,8 +186,11 @@ def attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m, eps: float, round_
 def latent_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m, eps: float) -> torch.Tensor:
     H, d, r, vd, rank = (int(m[k]) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank"))
     T = h.shape[0]
-    cq = rms(h @ w["dq"].T, eps) * w["dq.norm"]
-    q = (cq @ w["uq"].T).reshape(T, H, d + r)
+    if "dq" in w:
+        cq = rms(h @ w["dq"].T, eps) * w["dq.norm"]
+        q = (cq @ w["uq"].T).reshape(T, H, d + r)
+    else:
+        q = (h @ w["q"].T).reshape(T, H, d + r)
     dkv = h @ w["dkv"].T
     c = rms(dkv[:, :rank], eps) * w["dkv.norm"]
     kr = dkv[:, rank:].reshape(T, 1, r)
@@ -268,3 +272,14 @@ class PlainKegozen:
     def logits(self, tokens: Sequence[int]) -> torch.Tensor:
         x = self.layers_forward(tokens)[-1]
         return one_plus_norm(x, self.w["final.norm"], self.eps) @ self.w["head"].T
+
+    forward = logits
+
+    def greedy_generate(self, tokens: Sequence[int], count: int) -> List[int]:
+        """``count`` tokens, each the argmax (lowest index among equals) of the logits after all tokens before it."""
+        seq, out = list(tokens), []
+        for _ in range(count):
+            nxt = int(torch.argmax(self.logits(seq)[-1]))
+            out.append(nxt)
+            seq.append(nxt)
+        return out
