@@ -455,12 +455,39 @@ def tilivik_shape(size, layers, vocab):
     return cfg
 
 
+def kegozen_shape(size, layers, vocab):
+    """Layer sizes that resemble a real model's, for the Kegozen design: layers of a selective state-space mixer (inner
+    width twice the model's, heads of 64, a state of 128, 4 taps) alternate with windowed attention that sees older
+    positions as means of blocks (heads of 128 on the key/value heads of the Qwen2 model beside it, half of every head
+    turned with stretched wavelengths, values turned too, a window of 1,024 positions, blocks of 64) and with latent
+    attention over all positions (latents of 512 for keys and values and of half the width for queries); dense
+    feed-forwards alternate with scored experts and a gated shared expert."""
+    z = DESIGN_SIZES[size]
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            kind, mixer = "mamba2", dict(heads=2 * z["width"] // 64, vdim=64, state=128, groups=1, conv=4, norm_groups=1)
+        elif i % 4 == 1:
+            kind, mixer = "attention", dict(heads=z["heads"], kv_heads=max(2, z["heads"] // 7), dim=128, vdim=128, scale=128 ** -0.5,
+                                            rot=dict(base=1000000.0, dims=64, scaling=dict(factor=8.0, original=8192, fast=32.0, slow=1.0)),
+                                            mask=dict(size=1024, pool=64))
+        else:
+            kind, mixer = "latent_attention", dict(heads=z["heads"], dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=z["width"] // 2,
+                                                   scale=192 ** -0.5, rot=dict(base=10000.0, dims=64))
+        mlp = dict(kind="dense", ff=z["ff"]) if i % 2 == 0 else \
+            dict(kind="moe", expert=dict(ff=z["expert_ff"]), router=dict(experts=z["experts"], top=z["top"]),
+                 shared=dict(ff=z["expert_ff"]))
+        out.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    return dict(architecture="Kegozen", width=z["width"], vocab=vocab, norm=dict(eps=1e-6), layers=out)
+
+
 def design_comparison(args):
     """Prefill and decode of a model of the design at a real model's layer sizes, and of the benchmark's own
     architecture (Qwen2 dense) at the same width, layers, heads and dense feed-forward, one after the other; for
-    Tilivik also of Dedelorn, the nearest design the engine has (recurrent layers, a windowed attention, experts)."""
+    Tilivik and Kegozen also of Dedelorn, the nearest design the engine has (recurrent layers, latent attention,
+    experts)."""
     import torch
-    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig, TilivikConfig, TosisunConfig
+    from zedinfer_amd.config import DedelornConfig, KegozenConfig, Qwen2Config, SchedulerConfig, TilivikConfig, TosisunConfig
     from zedinfer_amd.engine import Engine
     layers = args.layers if args.layers != FULL_LAYERS else 8
     vocab, prompt = 32000, args.prompt_len
@@ -470,7 +497,8 @@ def design_comparison(args):
         z = DESIGN_SIZES[size]
         design = {"dedelorn": lambda: (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn"),
                   "tosisun": lambda: (TosisunConfig.from_dict(tosisun_shape(size, layers, vocab)), "Tosisun"),
-                  "tilivik": lambda: (TilivikConfig.from_dict(tilivik_shape(size, layers, vocab)), "Tilivik")}[args.design]
+                  "tilivik": lambda: (TilivikConfig.from_dict(tilivik_shape(size, layers, vocab)), "Tilivik"),
+                  "kegozen": lambda: (KegozenConfig.from_dict(kegozen_shape(size, layers, vocab)), "Kegozen")}[args.design]
         models = {
             args.design: design(),
             "qwen2": (Qwen2Config.from_dict(dict(SHAPE, hidden_size=z["width"], intermediate_size=z["ff"], vocab_size=vocab,
@@ -478,7 +506,7 @@ def design_comparison(args):
                                                  num_key_value_heads=max(2, z["heads"] // 7), tie_word_embeddings=False)),
                       "Qwen2ForCausalLM"),
         }
-        if args.design == "tilivik":
+        if args.design in ("tilivik", "kegozen"):
             models["dedelorn"] = (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn")
         if args.design_only:
             models = {args.design: models[args.design]}
@@ -535,7 +563,7 @@ def main():
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     ap.add_argument("--resident-layer", action="store_true",
                     help="instead: time the one-launch decoder layer (ops.decode_layer) alone, --layers launches a step")
-    ap.add_argument("--design", default="", choices=["", "dedelorn", "tosisun", "tilivik"],
+    ap.add_argument("--design", default="", choices=["", "dedelorn", "tosisun", "tilivik", "kegozen"],
                     help="instead: prefill and decode of a model of this design at a real model's layer sizes, beside "
                          "Qwen2 dense of equal sizes (8 layers unless --layers says otherwise)")
     ap.add_argument("--design-sizes", default="", help="with --design: layer sizes, of " + ", ".join(sorted(DESIGN_SIZES)) +

@@ -107,7 +107,8 @@ def _paged(T, ps, extra=3, seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,vd,rot,window,pool,ps,T", [
-    (4, 2, 32, 16, 16, 20, 4, 8, 70), (3, 3, 24, 24, 24, 33, 8, 4, 90), (5, 5, 20, 12, 10, 5, 7, 4, 40),
+    (4, 2, 32, 16, 16, 20, 4, 8, 70), (3, 3, 24, 24, 24, 33, 8, 4, 90), (12, 2, 128, 128, 64, 40, 8, 16, 200),
+    (6, 6, 64, 48, 64, 70, 32, 16, 210), (12, 1, 32, 32, 0, 16, 16, 8, 100), (2, 2, 96, 80, 32, 0, 0, 8, 75), (5, 5, 20, 12, 10, 5, 7, 4, 40),
     (2, 1, 8, 72, 0, 1, 3, 16, 30), (2, 1, 128, 96, 64, 50, 16, 16, 120), (4, 2, 16, 16, 8, 0, 0, 8, 45),
     (1, 1, 16, 8, 16, 12, 0, 8, 40)])
 def test_store_blocks_and_attention_against_the_plain_mechanism(dtype, H, G, d, vd, rot, window, pool, ps, T):
@@ -157,6 +158,7 @@ def test_store_blocks_and_attention_against_the_plain_mechanism(dtype, H, G, d, 
             if (j + 1) % pool == 0:
                 pslots[j] = prow_slots[j // pool]
     got = torch.zeros((T, H * vd), dtype=dtype, device=DEV)
+    cores_ran = [0]
     cuts = [T // 3, 1, T - T // 3 - 1]
     at = 0
     for n in cuts:
@@ -176,8 +178,20 @@ def test_store_blocks_and_attention_against_the_plain_mechanism(dtype, H, G, d, 
             ops.pool_blocks(kc, vc, kp, vp, _i32(pslots[at:at + n]), seqs, positions, table, G, d, vd, pool)
         ops.pooled_attention(qo, kc, vc, kp, vp, seqs, positions, table, ptab, H, G, d, vd, window, pool, scale,
                              out=got[at:at + n], vtable=vtab)
+        if ops.pooled_attention_cores_supported(dtype, H, G, d, vd):
+            # the matrix-core kernel on the same step: the entry as one portion, and beside two entries that it leaves
+            # alone (one too short, one of no tokens)
+            again = torch.full((n, H * vd), float("nan"), dtype=dtype, device=DEV)
+            wide = torch.cat([table, table, table])
+            wide_p = torch.cat([ptab, ptab, ptab]) if ptab is not None else None
+            ops.pooled_attention_cores(qo, kc, vc, kp, vp, _i32([0, 0, 0]), _i32([n, 1, 0]), _i32([at, at, 0]), n, wide, wide_p,
+                                       H, G, d, vd, window, pool, scale, out=again, vtable=vtab, long_len=min(n, 2))
+            _close(again.float(), got[at:at + n].float(), 2e-2, "matrix cores against the plain kernel")
+            cores_ran[0] += 1
         at += n
     _close(got.float().view(T, H, vd), want, 3e-4 if dtype == torch.float32 else 2e-2, "pooled attention")
+    if dtype == torch.bfloat16 and d in (32, 64, 96, 128) and vd % 16 == 0 and vd <= 128:
+        assert cores_ran[0] >= 2
 
 
 def test_a_far_block_that_carries_the_weight():

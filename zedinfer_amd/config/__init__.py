@@ -1,4 +1,4 @@
-from .model_config import ConfigError, DedelornConfig, ModelConfig, Qwen2Config, TilivikConfig, TosisunConfig, read_config_json
+from .model_config import ConfigError, DedelornConfig, KegozenConfig, ModelConfig, Qwen2Config, TilivikConfig, TosisunConfig, read_config_json
 from .forward_config import (LayerSpec, ModelForwardConfig, PartSpec, ScheduleStep,
                              default_schedule)
 from .registry import (Architecture, find_architecture, load_config, register_architecture,
@@ -6,7 +6,7 @@ from .registry import (Architecture, find_architecture, load_config, register_ar
 from .scheduler_config import SchedulerConfig
 
 __all__ = [
-    "ConfigError", "DedelornConfig", "ModelConfig", "Qwen2Config", "TilivikConfig", "TosisunConfig", "read_config_json", "LayerSpec",
+    "ConfigError", "DedelornConfig", "KegozenConfig", "ModelConfig", "Qwen2Config", "TilivikConfig", "TosisunConfig", "read_config_json", "LayerSpec",
     "ModelForwardConfig", "PartSpec", "ScheduleStep", "default_schedule", "Architecture",
     "find_architecture", "load_config", "register_architecture", "registered_architectures",
     "SchedulerConfig",

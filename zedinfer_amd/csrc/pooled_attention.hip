@@ -202,7 +202,9 @@ pooled_attention_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ 
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables, int max_pages,
                         int num_pages, int page_size, const int32_t* __restrict__ pool_tables, int pool_max_pages,
                         int pool_num_pages, int pool_page_size, int nh, int nkv, int dim, int vdim, int window, int pool,
-                        float scale, const float* __restrict__ vtable) {
+                        float scale, const float* __restrict__ vtable, const int32_t* __restrict__ entry_len, int long_len) {
+    // (the tokens of entries of long_len tokens and more are another kernel's)
+    if (entry_len && entry_len[tok_seq[blockIdx.x]] >= long_len) return;
     __shared__ float qs[PA_MAX_D];
     __shared__ float ps[PA_WAVES][ZI_WAVE];
     __shared__ int64_t vat[PA_WAVES][ZI_WAVE];
@@ -336,13 +338,15 @@ pooled_attention_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ 
 // `page_size` rows, found through block_tables [entries][max_pages]; block cache: kpool, vpool (float32) with
 // pool_num_pages pages of pool_page_size rows through pool_tables [entries][pool_max_pages] (null, or pool == 0: no
 // blocks, a plain window; window == 0: all positions, no blocks).  vtable [n][vdim/2][2] or null: the (cos, sin) of
-// every token's position over the value's pairs, by which a head's result is turned back.
+// every token's position over the value's pairs, by which a head's result is turned back.  entry_len (or null) and
+// long_len: the tokens of entries that bring long_len tokens or more are left out (the matrix-core kernel takes them).
 extern "C" int zi_pooled_attention(void* out, int64_t ldo, const void* q, int64_t ldq, int dt, const void* kcache,
                                    const void* vcache, const float* kpool, const float* vpool, const int32_t* tok_seq,
                                    const int32_t* tok_pos, const int32_t* block_tables, int max_pages, int num_pages,
                                    int page_size, const int32_t* pool_tables, int pool_max_pages, int pool_num_pages,
                                    int pool_page_size, int n, int nh, int nkv, int dim, int vdim, int window, int pool,
-                                   float scale, const float* vtable, hipStream_t stream) {
+                                   float scale, const float* vtable, const int32_t* entry_len, int long_len,
+                                   hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh <= 65535 && dim > 0 && vdim > 0 && dim <= PA_MAX_D &&
                    vdim <= PA_MAX_D, "pooled_attention: bad sizes (heads %d/%d, dim %d, vdim %d)", nh, nkv, dim, vdim);
     ZI_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0 && pool >= 0, "pooled_attention: bad cache sizes");
@@ -355,7 +359,7 @@ extern "C" int zi_pooled_attention(void* out, int64_t ldo, const void* q, int64_
         pooled_attention_kernel<T><<<dim3(n, nh), PA_WAVES * ZI_WAVE, 0, stream>>>(
             (T*)out, ldo, (const T*)q, ldq, (const T*)kcache, (const T*)vcache, kpool, vpool, tok_seq, tok_pos, block_tables,
             max_pages, num_pages, page_size, pool > 0 ? pool_tables : nullptr, pool_max_pages, pool_num_pages,
-            pool_page_size, nh, nkv, dim, vdim, window, pool, scale, vtable);
+            pool_page_size, nh, nkv, dim, vdim, window, pool, scale, vtable, entry_len, long_len);
     });
     return zi_check_launch("pooled_attention");
 }

@@ -280,7 +280,13 @@ int zi_pooled_attention(void* out, int64_t ldo, const void* q, int64_t ldq, int 
     vcache, const float* kpool, const float* vpool, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
     block_tables, int max_pages, int num_pages, int page_size, const int32_t* pool_tables, int pool_max_pages, int
     pool_num_pages, int pool_page_size, int n, int nh, int nkv, int dim, int vdim, int window, int pool, float scale,
-    const float* vtable, hipStream_t stream);
+    const float* vtable, const int32_t* entry_len, int long_len, hipStream_t stream);
+// pooled_attention_cores.hip
+int zi_pooled_attention_cores(void* out, int64_t ldo, const void* q, int64_t ldq, const void* kcache, const void*
+    vcache, const float* kpool, const float* vpool, const int32_t* entry_start, const int32_t* entry_len, const
+    int32_t* entry_past, int entries, int max_len, const int32_t* block_tables, int max_pages, int num_pages, int
+    page_size, const int32_t* pool_tables, int pool_max_pages, int pool_num_pages, int pool_page_size, int nh, int nkv,
+    int dim, int vdim, int window, int pool, float scale, const float* vtable, int long_len, hipStream_t stream);
 // norm.hip
 int zi_normed_add_norm(void* out, int out_dt, float* resid, const void* y, int y_dt, int64_t ldy, int splits, int64_t
     split_stride, const void* w1, const void* w2, int w_dt, int n, int hidden, float eps, float eps2, int add_one,
@@ -371,6 +377,7 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_norm_rope_store) \
     X(zi_pool_blocks) \
     X(zi_pooled_attention) \
+    X(zi_pooled_attention_cores) \
     X(zi_normed_add_norm) \
     X(zi_moe_route_sigmoid) \
     X(zi_moe_weighted_glu) \

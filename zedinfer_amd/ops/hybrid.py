@@ -202,11 +202,13 @@ def pooled_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                      vpool: Optional[torch.Tensor], tok_seq: torch.Tensor, positions: torch.Tensor,
                      block_tables: torch.Tensor, pool_tables: Optional[torch.Tensor], nh: int, nkv: int, dim: int,
                      vdim: int, window: int, pool: int, scale: float, out: torch.Tensor,
-                     vtable: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     vtable: Optional[torch.Tensor] = None, entry_len: Optional[torch.Tensor] = None,
+                     long_len: int = 0) -> torch.Tensor:
     """out [n, nh*vdim]: softmax attention of q [n, nh*dim] over the positions j with 0 <= i - j < window and over the
     means of the blocks of ``pool`` positions that lie wholly before the window (window 0: all positions; pool 0 or no
     ``pool_tables``: no blocks).  ``vtable`` [n, vdim/2, 2]: the (cos, sin) by which every head's result is turned
-    back (values were stored turned by their own positions)."""
+    back (values were stored turned by their own positions).  With ``entry_len`` and ``long_len`` the tokens of entries
+    that bring ``long_len`` tokens or more are left out (``pooled_attention_cores`` takes those)."""
     _gpu("pooled_attention", q, kcache, vcache, kpool, vpool, tok_seq, positions, block_tables, pool_tables, out, vtable)
     n = q.shape[0]
     ldq, wq = _rows(q, "pooled_attention q")
@@ -235,7 +237,59 @@ def pooled_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     _lib.call("zi_pooled_attention", _p(out), ldo, _p(q), ldq, _code(q, "pooled_attention q"), _p(kcache), _p(vcache),
               _p(kpool), _p(vpool), _p(tok_seq), _p(positions), _p(block_tables), int(block_tables.shape[1]), pages, ps,
               _p(pool_tables), pw, ppages, pps, n, nh, nkv, dim, vdim, int(window), int(pool if pool_tables is not None else 0),
-              float(scale), _p(vtable), _stream())
+              float(scale), _p(vtable), _p(entry_len), int(long_len), _stream())
+    return out
+
+
+def pooled_attention_cores_supported(dtype: torch.dtype, nh: int, nkv: int, dim: int, vdim: int) -> bool:
+    """Whether the matrix-core kernel takes these sizes (bfloat16; keys of 32, 64, 96 or 128 values, values of a
+    multiple of 16 up to 128; at most 64 query heads a key/value head)."""
+    if dtype != torch.bfloat16 or nkv <= 0:
+        return False
+    return bool(_lib.load().zi_pooled_attention_cores_supported(1, int(nh), int(nkv), int(dim), int(vdim)))
+
+
+def pooled_attention_cores(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, kpool: Optional[torch.Tensor],
+                           vpool: Optional[torch.Tensor], entry_start: torch.Tensor, entry_len: torch.Tensor,
+                           entry_past: torch.Tensor, max_len: int, block_tables: torch.Tensor,
+                           pool_tables: Optional[torch.Tensor], nh: int, nkv: int, dim: int, vdim: int, window: int,
+                           pool: int, scale: float, out: torch.Tensor, vtable: Optional[torch.Tensor] = None,
+                           long_len: int = 1) -> torch.Tensor:
+    """``pooled_attention`` on the matrix cores for the tokens of the entries that bring at least ``long_len`` tokens
+    (``max_len``: the most any entry brings); the rows of other tokens are not written."""
+    _gpu("pooled_attention_cores", q, kcache, vcache, kpool, vpool, entry_start, entry_len, entry_past, block_tables,
+         pool_tables, out, vtable)
+    n = q.shape[0]
+    ldq, wq = _rows(q, "pooled_attention_cores q")
+    ldo, wo = _rows(out, "pooled_attention_cores out")
+    if not pooled_attention_cores_supported(q.dtype, nh, nkv, dim, vdim):
+        raise ValueError("pooled_attention_cores: sizes or a type the kernel does not take")
+    if wq != nh * dim or wo != nh * vdim or out.shape[0] != n or kcache.dtype != q.dtype or out.dtype != q.dtype:
+        raise ValueError("pooled_attention_cores: q [n, nh*dim] and out [n, nh*vdim] in the cache's type")
+    pages, ps = _token_cache(kcache, vcache, nkv, dim, vdim, "pooled_attention_cores")
+    E = entry_start.numel()
+    for t in (entry_start, entry_len, entry_past):
+        _i32(t, "pooled_attention_cores entries", E)
+    _i32(block_tables, "pooled_attention_cores block_tables")
+    if block_tables.dim() != 2 or block_tables.shape[0] < E:
+        raise ValueError("pooled_attention_cores: one row of the block table an entry")
+    ppages = pps = pw = 0
+    if pool_tables is not None and pool > 0:
+        if kpool is None or vpool is None or kpool.dtype != torch.float32 or vpool.dtype != torch.float32:
+            raise ValueError("pooled_attention_cores: blocks need their float32 means")
+        ppages, pps = _token_cache(kpool, vpool, nkv, dim, vdim, "pooled_attention_cores means")
+        _i32(pool_tables, "pooled_attention_cores pool_tables")
+        if pool_tables.shape[0] != block_tables.shape[0]:
+            raise ValueError("pooled_attention_cores: one row of either table an entry")
+        pw = int(pool_tables.shape[1])
+    else:
+        pool_tables = None
+    if vtable is not None:
+        _f32(vtable, "pooled_attention_cores vtable", (n, vdim // 2, 2))
+    _lib.call("zi_pooled_attention_cores", _p(out), ldo, _p(q), ldq, _p(kcache), _p(vcache), _p(kpool), _p(vpool),
+              _p(entry_start), _p(entry_len), _p(entry_past), E, int(max_len), _p(block_tables), int(block_tables.shape[1]),
+              pages, ps, _p(pool_tables), pw, ppages, pps, nh, nkv, dim, vdim, int(window),
+              int(pool if pool_tables is not None else 0), float(scale), _p(vtable), int(long_len), _stream())
     return out
 
 

@@ -71,6 +71,9 @@ class PooledWindowAttention(Mixer):
     tape_safe = True
     padding_safe = True      # padding has no place in either cache and no real token sees it
     writes_into = True
+    # entries that bring at least this many tokens (portions of prompts) go to the matrix-core kernel, where it takes
+    # the sizes; decoded tokens and short portions to the kernel that deals a token's keys over four wavefronts
+    LONG_ENTRY = 8
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -121,6 +124,7 @@ class PooledWindowAttention(Mixer):
         stacked = torch.zeros((-(-width // 8) * 8, self.hidden), dtype=q.dtype, device=q.device)     # rows to a multiple of 8
         stacked[:width] = torch.cat([q, k.to(q.dtype), v.to(q.dtype)])
         self.qkv, self.width, self.o = stacked, width, o.contiguous()
+        self.cores = rt.device.type == "cuda" and ops.pooled_attention_cores_supported(rt.dtype, self.nh, self.nkv, self.d, self.vd)
         self.table_key = self.vtable_key = None
         if self.rot:
             theta, scaling = float(p["theta"]), p.get("scaling")
@@ -178,8 +182,16 @@ class PooledWindowAttention(Mixer):
                 ops.pool_blocks(kc, vc, kp, vp, bview.slots, batch.tok_seq, batch.positions, view.block_tables, self.nkv,
                                 self.d, self.vd, self.pool)
         heads = rt.buffer("pooled_heads", (n, self.nh * self.vd))
-        ops.pooled_attention(q, kc, vc, kp, vp, batch.tok_seq, batch.positions, view.block_tables, ptab, self.nh, self.nkv,
-                             self.d, self.vd, self.window, self.pool, self.scale, out=heads, vtable=vtable)
+        lens = batch.host_len
+        longest = int(lens.max()) if self.cores and lens is not None else 0
+        if longest >= self.LONG_ENTRY:
+            ops.pooled_attention_cores(q, kc, vc, kp, vp, batch.entry_start, batch.entry_len, batch.entry_past, longest,
+                                       view.block_tables, ptab, self.nh, self.nkv, self.d, self.vd, self.window, self.pool,
+                                       self.scale, out=heads, vtable=vtable, long_len=self.LONG_ENTRY)
+        if longest < self.LONG_ENTRY or int(lens.min()) < self.LONG_ENTRY:
+            ops.pooled_attention(q, kc, vc, kp, vp, batch.tok_seq, batch.positions, view.block_tables, ptab, self.nh, self.nkv,
+                                 self.d, self.vd, self.window, self.pool, self.scale, out=heads, vtable=vtable,
+                                 entry_len=batch.entry_len if longest >= self.LONG_ENTRY else None, long_len=self.LONG_ENTRY)
         if out is None:
             out = rt.buffer("pooled_out", (n, self.hidden))
         return ops.linear(heads, self.o, out=out)
