@@ -159,7 +159,7 @@ def test_store_blocks_and_attention_against_the_plain_mechanism(dtype, H, G, d, 
                 pslots[j] = prow_slots[j // pool]
     got = torch.zeros((T, H * vd), dtype=dtype, device=DEV)
     cores_ran = [0]
-    cuts = [T // 3, 1, T - T // 3 - 1]
+    cuts = [T // 3, 1, 3, T - T // 3 - 4]
     at = 0
     for n in cuts:
         positions = _i32(list(range(at, at + n)))
@@ -188,6 +188,18 @@ def test_store_blocks_and_attention_against_the_plain_mechanism(dtype, H, G, d, 
                                        H, G, d, vd, window, pool, scale, out=again, vtable=vtab, long_len=min(n, 2))
             _close(again.float(), got[at:at + n].float(), 2e-2, "matrix cores against the plain kernel")
             cores_ran[0] += 1
+            if n <= 64 // (H // G):
+                # ... and as a short entry: its items cut into chunks over workgroups, merged by the second kernel
+                for max_keys in (at + n, at + n + 300):
+                    chunks, per = ops.pooled_attention_cores_cut(max_keys, window, pool, n, 256, G)
+                    ws = torch.full((ops.pooled_attention_cores_workspace(n, H, vd, chunks),), float("nan"), device=DEV)
+                    again = torch.full((n, H * vd), float("nan"), dtype=dtype, device=DEV)
+                    ops.pooled_attention_cores(qo, kc, vc, kp, vp, _i32([0, 0]), _i32([n, 0]), _i32([at, 0]), n, wide[:2],
+                                               wide_p[:2] if wide_p is not None else None, H, G, d, vd, window, pool, scale,
+                                               out=again, vtable=vtab, long_len=n + 1, chunks=chunks, chunk_blocks=per,
+                                               workspace=ws, tok_seq=seqs)
+                    _close(again.float(), got[at:at + n].float(), 2e-2, "keys cut over workgroups against the plain kernel")
+                cores_ran[0] += 1
         at += n
     _close(got.float().view(T, H, vd), want, 3e-4 if dtype == torch.float32 else 2e-2, "pooled attention")
     if dtype == torch.bfloat16 and d in (32, 64, 96, 128) and vd % 16 == 0 and vd <= 128:

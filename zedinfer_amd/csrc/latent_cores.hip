@@ -280,7 +280,8 @@ extern "C" int zi_latent_attention_cores(float* out, float* partial, int64_t par
     if (chunks > 1) {
         // every key a tile's rows see lies in one of the chunks
         const int tokens_in_tile = (16 * waves + heads - 1) / heads + 1;
-        ZI_REQUIRE(window > 0 && (int64_t)chunks * chunk_keys >= (int64_t)window + tokens_in_tile,
+        // (without a window the caller sees to it that the chunks reach the last key of every entry)
+        ZI_REQUIRE(window == 0 || (int64_t)chunks * chunk_keys >= (int64_t)window + tokens_in_tile,
                    "latent_attention_cores: %d chunks of %d keys do not cover a window of %d", chunks, chunk_keys, window);
         ZI_REQUIRE(partial && partial_floats >= (int64_t)chunks * n * heads * (rank + 2),
                    "latent_attention_cores: the workspace is too small");

@@ -38,17 +38,22 @@ pooled_attention_cores_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_b
                               const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
                               int max_pages, int num_pages, int page_size, const int32_t* __restrict__ pool_tables,
                               int pool_max_pages, int pool_num_pages, int pool_page_size, int nh, int nkv, int window,
-                              int pool, float scale_log2, const float* __restrict__ vtable, int long_len) {
+                              int pool, float scale_log2, const float* __restrict__ vtable, int long_len,
+                              int chunk_blocks, float* __restrict__ partial, int total_rows) {
     constexpr int DIM = 32 * DK32, VD = 16 * DV16, KS = DIM + 8;
     __shared__ __attribute__((aligned(16))) uint16_t ks[PC_ITEMS][KS];
     __shared__ __attribute__((aligned(16))) uint16_t vt[VD][PC_VT_STRIDE];
     __shared__ __attribute__((aligned(16))) float os[PC_ROWS][VD + 1];
     const int e = blockIdx.z, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int len = entry_len[e];
-    if (len < long_len) return;
     const int group = nh / nkv;
     const int tq_tile = PC_ROWS / group;           // tokens a tile holds
-    const int tq0 = blockIdx.x * tq_tile;
+    // chunk_blocks > 0: the short entries (fewer than long_len tokens: one tile), their items cut into chunks of
+    // chunk_blocks blocks over blockIdx.x, the chunks' unnormalised results left in `partial`; else the long ones,
+    // a tile a workgroup
+    const bool split = chunk_blocks > 0;
+    if (split ? (len >= long_len || len <= 0) : len < long_len) return;
+    const int tq0 = split ? 0 : blockIdx.x * tq_tile;
     if (tq0 >= len) return;
     const int tq_n = len - tq0 < tq_tile ? len - tq0 : tq_tile;
     const int past = entry_past[e], t0 = entry_start[e] + tq0;
@@ -81,7 +86,10 @@ pooled_attention_cores_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_b
     float m_run = -1e30f, l_run = 0.f;
 
     const int blocks_pool = (nb_max + PC_ITEMS - 1) / PC_ITEMS, blocks_tok = (n_tok + PC_ITEMS - 1) / PC_ITEMS;
-    for (int blk = 0; blk < blocks_pool + blocks_tok; ++blk) {
+    const int blk_first = split ? blockIdx.x * chunk_blocks : 0;
+    const int blk_end = split && blk_first + chunk_blocks < blocks_pool + blocks_tok ? blk_first + chunk_blocks
+                                                                                     : blocks_pool + blocks_tok;
+    for (int blk = blk_first; blk < blk_end; ++blk) {
         const bool pool_phase = blk < blocks_pool;
         const int base = pool_phase ? blk * PC_ITEMS : (blk - blocks_pool) * PC_ITEMS;
         const int n_items = pool_phase ? nb_max : n_tok;
@@ -197,6 +205,22 @@ pooled_attention_cores_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_b
     float l_row = l_run;
     l_row += __shfl_xor(l_row, 16, ZI_WAVE);
     l_row += __shfl_xor(l_row, 32, ZI_WAVE);
+    if (split) {
+        // this chunk's share of the row: (maximum in base-2 units, sum, unnormalised result); a chunk without
+        // items leaves a share that counts nothing
+        if (r_ok) {
+            float* dst = partial + ((int64_t)blockIdx.x * total_rows + (int64_t)(t0 + r_tok) * nh + g * group + r_head) * (VD + 2);
+            if (j == 0) {
+                dst[0] = m_run;
+                dst[1] = l_row;
+            }
+#pragma unroll
+            for (int v = 0; v < DV16; ++v)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) dst[2 + 16 * v + 4 * j + i] = acc_o[v][i];
+        }
+        return;
+    }
     const float inv = l_row > 0.f ? 1.f / l_row : 0.f;
 #pragma unroll
     for (int v = 0; v < DV16; ++v)
@@ -218,20 +242,65 @@ pooled_attention_cores_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_b
     }
 }
 
+// The rows of the short entries from their chunks' shares, in rising order of the chunks; turned back where values
+// are stored turned.  One workgroup per (token, head); tokens of long entries are left alone.
+__global__ void __launch_bounds__(128)
+pooled_attention_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const float* __restrict__ partial, int chunks,
+                              int total_rows, int nh, int vd, const float* __restrict__ vtable,
+                              const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ entry_len, int long_len) {
+    __shared__ float os[128];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int len = entry_len[tok_seq[t]];
+    if (len >= long_len) return;
+    const int64_t row = (int64_t)t * nh + h;
+    float M = -1e30f;
+    for (int c = 0; c < chunks; ++c) M = fmaxf(M, partial[((int64_t)c * total_rows + row) * (vd + 2)]);
+    float L = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+        const float* p = partial + ((int64_t)c * total_rows + row) * (vd + 2);
+        L += p[1] * exp2f(p[0] - M);
+    }
+    const int x = threadIdx.x;
+    if (x < vd) {
+        float o = 0.f;
+        for (int c = 0; c < chunks; ++c) {
+            const float* p = partial + ((int64_t)c * total_rows + row) * (vd + 2);
+            o += p[2 + x] * exp2f(p[0] - M);
+        }
+        os[x] = L > 0.f ? o / L : 0.f;
+    }
+    __syncthreads();
+    if (x < vd) {
+        float o = os[x];
+        const int vh = vd / 2;
+        if (vtable) {
+            const int pr = x < vh ? x : x - vh;
+            const float cs = vtable[((int64_t)t * vh + pr) * 2], sn = vtable[((int64_t)t * vh + pr) * 2 + 1];
+            o = x < vh ? os[x] * cs + os[x + vh] * sn : os[x] * cs - os[x - vh] * sn;
+        }
+        zi_store(out + (int64_t)t * ldo + (int64_t)h * vd + x, o);
+    }
+}
+
 extern "C" int zi_pooled_attention_cores_supported(int dt, int nh, int nkv, int dim, int vdim) {
     return dt == ZI_BF16 && nkv > 0 && nh % nkv == 0 && nh / nkv <= PC_ROWS && (dim == 32 || dim == 64 || dim == 96 || dim == 128) &&
            vdim % 16 == 0 && vdim >= 16 && vdim <= 128;
 }
 
 // The entries of at least `long_len` tokens of this step; `max_len` is the most tokens an entry brings (it sizes the
-// launch).  Everything else as zi_pooled_attention.
+// launch).  Everything else as zi_pooled_attention.  With chunks > 0 instead the entries of FEWER than long_len tokens
+// (long_len - 1 tokens times the heads of a group must fit 64 rows): every entry's items are cut into `chunks` chunks
+// of chunk_blocks blocks of 32 (the caller sees to it that they cover the items of every such entry), whose shares go
+// through `partial` (chunks * n * nh * (vdim + 2) floats) and a second kernel; tok_seq [n] names every token's entry.
 extern "C" int zi_pooled_attention_cores(void* out, int64_t ldo, const void* q, int64_t ldq, const void* kcache,
                                          const void* vcache, const float* kpool, const float* vpool,
                                          const int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_past,
                                          int entries, int max_len, const int32_t* block_tables, int max_pages, int num_pages,
                                          int page_size, const int32_t* pool_tables, int pool_max_pages, int pool_num_pages,
                                          int pool_page_size, int nh, int nkv, int dim, int vdim, int window, int pool,
-                                         float scale, const float* vtable, int long_len, hipStream_t stream) {
+                                         float scale, const float* vtable, int long_len, int chunks, int chunk_blocks,
+                                         float* partial, int64_t partial_floats, const int32_t* tok_seq, int n,
+                                         hipStream_t stream) {
     ZI_REQUIRE(zi_pooled_attention_cores_supported(ZI_BF16, nh, nkv, dim, vdim), "pooled_attention_cores: sizes it does not take "
                "(heads %d/%d, dim %d, vdim %d)", nh, nkv, dim, vdim);
     ZI_REQUIRE(entries >= 0 && entries <= 65535 && nkv <= 65535 && max_len >= 0 && page_size > 0 && max_pages > 0 && num_pages > 0 &&
@@ -240,15 +309,25 @@ extern "C" int zi_pooled_attention_cores(void* out, int64_t ldo, const void* q, 
                "pooled_attention_cores: blocks without a cache of their means");
     ZI_REQUIRE(ldq >= (int64_t)nh * dim && ldo >= (int64_t)nh * vdim && ldq % 8 == 0 && ((uintptr_t)q % 16) == 0 &&
                ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0, "pooled_attention_cores: rows must be 16-byte aligned");
-    if (entries == 0 || max_len < long_len) return 0;
     const int tq_tile = PC_ROWS / (nh / nkv);
-    const dim3 grid((max_len + tq_tile - 1) / tq_tile, nkv, entries);
+    const bool split = chunks > 0;
+    if (split) {
+        ZI_REQUIRE(chunk_blocks > 0 && chunks <= 65535 && long_len - 1 <= tq_tile && tok_seq && n >= 0,
+                   "pooled_attention_cores: a bad cut (%d chunks of %d blocks, entries below %d tokens)", chunks, chunk_blocks, long_len);
+        ZI_REQUIRE(partial && partial_floats >= (int64_t)chunks * n * nh * (vdim + 2), "pooled_attention_cores: the workspace is too small");
+        if (entries == 0 || n == 0) return 0;
+    } else if (entries == 0 || max_len < long_len) {
+        return 0;
+    }
+    const dim3 grid(split ? chunks : (max_len + tq_tile - 1) / tq_tile, nkv, entries);
+    const int total_rows = n * nh;
     const float scale_log2 = scale * 1.4426950408889634f;
 #define ZI_PC(DK32, DV16)                                                                                              \
     pooled_attention_cores_kernel<DK32, DV16><<<grid, PC_THREADS, 0, stream>>>(                                        \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, kpool, vpool,      \
         entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, page_size, pool > 0 ? pool_tables : nullptr, \
-        pool_max_pages, pool_num_pages, pool_page_size, nh, nkv, window, pool, scale_log2, vtable, long_len)
+        pool_max_pages, pool_num_pages, pool_page_size, nh, nkv, window, pool, scale_log2, vtable, long_len,           \
+        split ? chunk_blocks : 0, partial, total_rows)
 #define ZI_PC_V(DK32)                                   \
     switch (vdim / 16) {                                \
         case 1: ZI_PC(DK32, 1); break;                  \
@@ -268,5 +347,9 @@ extern "C" int zi_pooled_attention_cores(void* out, int64_t ldo, const void* q, 
     }
 #undef ZI_PC_V
 #undef ZI_PC
-    return zi_check_launch("pooled_attention_cores");
+    const int rc = zi_check_launch("pooled_attention_cores");
+    if (rc != 0 || !split) return rc;
+    pooled_attention_merge_kernel<<<dim3(n, nh), 128, 0, stream>>>((zi_bf16*)out, ldo, partial, chunks, total_rows, nh, vdim,
+                                                                  vtable, tok_seq, entry_len, long_len);
+    return zi_check_launch("pooled_attention_merge");
 }

@@ -286,7 +286,8 @@ int zi_pooled_attention_cores(void* out, int64_t ldo, const void* q, int64_t ldq
     vcache, const float* kpool, const float* vpool, const int32_t* entry_start, const int32_t* entry_len, const
     int32_t* entry_past, int entries, int max_len, const int32_t* block_tables, int max_pages, int num_pages, int
     page_size, const int32_t* pool_tables, int pool_max_pages, int pool_num_pages, int pool_page_size, int nh, int nkv,
-    int dim, int vdim, int window, int pool, float scale, const float* vtable, int long_len, hipStream_t stream);
+    int dim, int vdim, int window, int pool, float scale, const float* vtable, int long_len, int chunks, int
+    chunk_blocks, float* partial, int64_t partial_floats, const int32_t* tok_seq, int n, hipStream_t stream);
 // norm.hip
 int zi_normed_add_norm(void* out, int out_dt, float* resid, const void* y, int y_dt, int64_t ldy, int splits, int64_t
     split_stride, const void* w1, const void* w2, int w_dt, int n, int hidden, float eps, float eps2, int add_one,

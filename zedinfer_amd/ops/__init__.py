@@ -29,7 +29,8 @@ from .recurrent import (attention_biased, embedding_sum, gate_heads, gated_rms_n
                         token_shift)
 from . import hybrid
 from .hybrid import (linear_attention_grouped, moe_route_sigmoid, moe_sum_shared, moe_weighted_glu, norm_rope_store,
-                     normed_add_norm, pool_blocks, pooled_attention, pooled_attention_cores, pooled_attention_cores_supported,
+                     normed_add_norm, pool_blocks, pooled_attention, pooled_attention_cores, pooled_attention_cores_cut, pooled_attention_cores_supported,
+                     pooled_attention_cores_workspace,
                      rope_table_scaled, ssm_finish, ssm_prepare,
                      ssm_state_floats)
 from ._lib import KernelLibraryError, library_path, load
@@ -54,6 +55,6 @@ __all__ = [
     "attention_biased", "embedding_sum", "gate_heads", "gated_rms_norm_act", "linear_attention",
     "linear_attention_state_floats", "lowrank_decay", "moe_route_table", "normed_kv_store", "stream_reenter", "token_shift",
     "linear_attention_grouped", "moe_route_sigmoid", "moe_sum_shared", "moe_weighted_glu", "norm_rope_store",
-    "normed_add_norm", "pool_blocks", "pooled_attention", "pooled_attention_cores", "pooled_attention_cores_supported", "rope_table_scaled", "ssm_finish", "ssm_prepare", "ssm_state_floats",
+    "normed_add_norm", "pool_blocks", "pooled_attention", "pooled_attention_cores", "pooled_attention_cores_cut", "pooled_attention_cores_supported", "pooled_attention_cores_workspace", "rope_table_scaled", "ssm_finish", "ssm_prepare", "ssm_state_floats",
     "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

@@ -118,7 +118,8 @@ _PROTOTYPES = {
     "zi_norm_rope_store": [P, I, L, P, P, P, L, I, L, P, P, F, P, I, P, P, L, I, I, I, I, I, P],
     "zi_pool_blocks": [P, P, L, P, P, I, P, P, P, P, I, I, I, I, I, I, I, I, P],
     "zi_pooled_attention": [P, L, P, L, I, P, P, P, P, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, I, F, P, P, I, P],
-    "zi_pooled_attention_cores": [P, L, P, L, P, P, P, P, P, P, P, I, I, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I, P],
+    "zi_pooled_attention_cores": [P, L, P, L, P, P, P, P, P, P, P, I, I, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I,
+                                  I, I, P, L, P, I, P],
     "zi_pooled_attention_cores_supported": [I, I, I, I, I],
     "zi_normed_add_norm": [P, I, P, P, I, L, I, L, P, P, I, I, I, F, F, I, P],
     "zi_moe_route_sigmoid": [P, P, P, L, I, I, I, P],

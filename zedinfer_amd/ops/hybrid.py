@@ -254,9 +254,14 @@ def pooled_attention_cores(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.
                            entry_past: torch.Tensor, max_len: int, block_tables: torch.Tensor,
                            pool_tables: Optional[torch.Tensor], nh: int, nkv: int, dim: int, vdim: int, window: int,
                            pool: int, scale: float, out: torch.Tensor, vtable: Optional[torch.Tensor] = None,
-                           long_len: int = 1) -> torch.Tensor:
+                           long_len: int = 1, chunks: int = 0, chunk_blocks: int = 0,
+                           workspace: Optional[torch.Tensor] = None, tok_seq: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``pooled_attention`` on the matrix cores for the tokens of the entries that bring at least ``long_len`` tokens
-    (``max_len``: the most any entry brings); the rows of other tokens are not written."""
+    (``max_len``: the most any entry brings); the rows of other tokens are not written.  With ``chunks`` > 0 instead
+    for the entries that bring FEWER than ``long_len`` tokens (decoded tokens): the items every such entry sees (the
+    blocks, then the window's positions) are cut into ``chunks`` chunks of ``chunk_blocks`` blocks of 32 items over
+    workgroups and merged by a second kernel through ``workspace`` (``pooled_attention_cores_workspace`` floats);
+    the caller chooses the cut so that it covers every entry's items (``pooled_attention_cores_cut``)."""
     _gpu("pooled_attention_cores", q, kcache, vcache, kpool, vpool, entry_start, entry_len, entry_past, block_tables,
          pool_tables, out, vtable)
     n = q.shape[0]
@@ -286,11 +291,43 @@ def pooled_attention_cores(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.
         pool_tables = None
     if vtable is not None:
         _f32(vtable, "pooled_attention_cores vtable", (n, vdim // 2, 2))
+    if chunks > 0:
+        need = pooled_attention_cores_workspace(n, nh, vdim, chunks)
+        if workspace is None or workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+            raise ValueError(f"pooled_attention_cores: {need} floats of workspace are needed")
+        if tok_seq is None or chunk_blocks <= 0 or (long_len - 1) * (nh // nkv) > POOLED_ROWS:
+            raise ValueError("pooled_attention_cores: a cut needs every token's entry, blocks a chunk, and short entries that fit a tile")
+        _i32(tok_seq, "pooled_attention_cores tok_seq", n)
     _lib.call("zi_pooled_attention_cores", _p(out), ldo, _p(q), ldq, _p(kcache), _p(vcache), _p(kpool), _p(vpool),
               _p(entry_start), _p(entry_len), _p(entry_past), E, int(max_len), _p(block_tables), int(block_tables.shape[1]),
               pages, ps, _p(pool_tables), pw, ppages, pps, nh, nkv, dim, vdim, int(window),
-              int(pool if pool_tables is not None else 0), float(scale), _p(vtable), int(long_len), _stream())
+              int(pool if pool_tables is not None else 0), float(scale), _p(vtable), int(long_len), int(chunks),
+              int(chunk_blocks), _p(workspace), int(workspace.numel()) if workspace is not None else 0, _p(tok_seq), n, _stream())
     return out
+
+
+POOLED_ITEMS = 32          # items (blocks' means or positions) a block of the matrix-core kernel holds
+POOLED_ROWS = 64           # rows (token, head of a group) a workgroup of it holds
+
+
+def pooled_attention_cores_cut(max_keys: int, window: int, pool: int, most_tokens: int, units: int, tiles: int):
+    """(chunks, blocks a chunk) for the short entries of a step none of which holds more than ``max_keys`` tokens
+    once it has run and brings more than ``most_tokens``: chunks of four blocks of 32 items, of more when ``tiles``
+    (entries x key/value heads) workgroups a chunk would be many more than the chip holds at a time."""
+    if window > 0:
+        span = min(window + most_tokens, max_keys)
+        means = -(-(max_keys // pool) // POOLED_ITEMS) if pool > 0 else 0
+        blocks = means + -(-span // POOLED_ITEMS) + 1     # the positions' first block starts anywhere
+    else:
+        blocks = -(-max_keys // POOLED_ITEMS)
+    per = 4
+    while per < blocks and -(-blocks // per) * max(tiles, 1) > 4 * max(units, 1):
+        per *= 2
+    return max(1, -(-blocks // per)), per
+
+
+def pooled_attention_cores_workspace(n: int, nh: int, vdim: int, chunks: int) -> int:
+    return int(chunks) * int(n) * int(nh) * (int(vdim) + 2)
 
 
 # ---- a norm on a sublayer's output -----------------------------------------------------------------------------

@@ -154,10 +154,11 @@ def latent_attention_cores_supported(cache_dtype: torch.dtype, rank: int, rot: i
     return bool(_lib.load().zi_latent_attention_cores_supported(1, int(rank), int(rot)))
 
 
-def latent_attention_cores_plan(n: int, entries: int, heads: int, window: int, units: int):
+def latent_attention_cores_plan(n: int, entries: int, heads: int, window: int, units: int, max_keys: int = 0):
     """(wavefronts a workgroup, keys a chunk, chunks) for a step of n tokens in ``entries`` entries: 64 rows a
     workgroup when that many tiles fill the chip, else 16; a tile's keys are cut into chunks when the tiles alone
-    are fewer than the chip's compute units (decoded tokens, short portions) and a window bounds them.  A function of the step's shape."""
+    are fewer than the chip's compute units (decoded tokens, short portions) and a window bounds them, or, without
+    a window, ``max_keys`` does (no entry holds more tokens once the step has run).  A function of the step's shape."""
     lib = _lib.load()
     waves = 4 if lib.zi_latent_attention_cores_tiles(int(n), int(entries), int(heads), 4) >= units else 1
     tiles = lib.zi_latent_attention_cores_tiles(int(n), int(entries), int(heads), waves)
@@ -166,6 +167,13 @@ def latent_attention_cores_plan(n: int, entries: int, heads: int, window: int, u
         chunks = -(-span // LATENT_CHUNK_KEYS)
         if chunks > 1:
             return waves, LATENT_CHUNK_KEYS, chunks
+    if window <= 0 and max_keys > 0 and tiles < units:
+        keys = LATENT_CHUNK_KEYS
+        while -(-int(max_keys) // keys) * tiles > 4 * units:      # no more workgroups than four rounds of the chip
+            keys *= 2
+        chunks = -(-int(max_keys) // keys)
+        if chunks > 1:
+            return waves, keys, chunks
     return waves, 0, 1
 
 

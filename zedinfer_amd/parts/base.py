@@ -292,6 +292,31 @@ class StepPlanner:
         return tuple(sorted(int(n) for n in entry_lens))
 
 
+class KeyBoundPlanner(StepPlanner):
+    """For mixers whose launches are sized by the most keys a token of the step can see and nothing else: the plan
+    has no arrays and one size, ``max_keys``, at least the tokens any entry holds once the step has run: the engine's
+    recurring bounds when it gives them (steps that are replayed), the exact number otherwise."""
+
+    key = ("key_bound",)
+    fixed_for_single_tokens = True
+
+    def plan(self, hb: HostBatch) -> StepPlan:
+        lens, ends = hb.entry_len, hb.entry_past + hb.entry_len
+        single = lens == 1
+        bound = 0
+        if single.any():
+            bound = max(bound, int(hb.bound_single) or int(ends[single].max()))
+        if (~single).any():
+            bound = max(bound, int(hb.bound_multi) or int(ends[~single].max()))
+        return StepPlan(sizes={"max_keys": max(bound, 1)})
+
+    def shape(self, entry_lens, bound_single: int, bound_multi: int) -> tuple:
+        return ()
+
+
+KEY_BOUND_PLANNER = KeyBoundPlanner()
+
+
 class Mixer(Part):
     """Mixes information across the tokens of a sequence.
 

@@ -8,7 +8,8 @@ import torch
 from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
-from .base import (PAGE, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime, register_mixer)
+from .base import (KEY_BOUND_PLANNER, PAGE, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime,
+                   StepPlanner, register_mixer)
 from .rows import ProductRows
 
 
@@ -118,6 +119,10 @@ class LatentAttention(Mixer):
     def step_rows(self, rows: int, kind: str) -> int:
         return ProductRows.step_rows(rows, kind)
 
+    def planner(self) -> Optional[StepPlanner]:
+        """Without a window the cut of a tile's keys over workgroups is sized by the most keys a token sees."""
+        return KEY_BOUND_PLANNER if self.window <= 0 else None
+
     def forward(self, x: torch.Tensor, batch, memory: LayerMemory, out=None) -> torch.Tensor:
         n, rt = x.shape[0], self.rt
         view = batch.groups[memory.group]
@@ -136,7 +141,9 @@ class LatentAttention(Mixer):
         ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa, w_uk_t=self.uk_t)
         o = rt.buffer("latent_attended", (n, self.nh, self.rank), torch.float32)
         if self.cores:
-            waves, chunk_keys, chunks = ops.latent_attention_cores_plan(n, batch.num_entries, self.nh, self.window, self.units)
+            max_keys = batch.plans[KEY_BOUND_PLANNER.key].sizes["max_keys"] if self.window <= 0 else 0
+            waves, chunk_keys, chunks = ops.latent_attention_cores_plan(n, batch.num_entries, self.nh, self.window, self.units,
+                                                                        max_keys=max_keys)
             need = ops.latent_attention_cores_workspace(n, self.nh, self.rank, chunks)
             ws = rt.buffer("latent_chunks", (need,), torch.float32) if need else None
             ops.latent_attention_cores(qa, c_cache, kr_cache, batch.entry_start, batch.entry_len, batch.entry_past,

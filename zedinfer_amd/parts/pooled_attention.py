@@ -10,7 +10,7 @@ import torch
 from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
-from .base import PAGE, KVCacheRequest, LayerMemory, Mixer, PageTensor, Runtime, register_mixer
+from .base import KEY_BOUND_PLANNER, PAGE, KVCacheRequest, LayerMemory, Mixer, PageTensor, Runtime, StepPlanner, register_mixer
 from .rows import ProductRows
 
 
@@ -71,8 +71,9 @@ class PooledWindowAttention(Mixer):
     tape_safe = True
     padding_safe = True      # padding has no place in either cache and no real token sees it
     writes_into = True
-    # entries that bring at least this many tokens (portions of prompts) go to the matrix-core kernel, where it takes
-    # the sizes; decoded tokens and short portions to the kernel that deals a token's keys over four wavefronts
+    # Where the matrix-core kernel takes the sizes: entries that bring at least this many tokens (portions of prompts)
+    # a tile of queries a workgroup; shorter ones (decoded tokens), which fit one tile, with their keys cut over
+    # workgroups and merged.  Everything else goes to the kernel that deals a token's keys over four wavefronts.
     LONG_ENTRY = 8
 
     @staticmethod
@@ -125,6 +126,8 @@ class PooledWindowAttention(Mixer):
         stacked[:width] = torch.cat([q, k.to(q.dtype), v.to(q.dtype)])
         self.qkv, self.width, self.o = stacked, width, o.contiguous()
         self.cores = rt.device.type == "cuda" and ops.pooled_attention_cores_supported(rt.dtype, self.nh, self.nkv, self.d, self.vd)
+        self.long_entry = min(self.LONG_ENTRY, ops.hybrid.POOLED_ROWS // (self.nh // self.nkv) + 1)
+        self.units = ops.compute_units() if rt.device.type == "cuda" else 256
         self.table_key = self.vtable_key = None
         if self.rot:
             theta, scaling = float(p["theta"]), p.get("scaling")
@@ -153,6 +156,9 @@ class PooledWindowAttention(Mixer):
 
     def step_rows(self, rows: int, kind: str) -> int:
         return ProductRows.step_rows(rows, kind)
+
+    def planner(self) -> Optional[StepPlanner]:
+        return KEY_BOUND_PLANNER
 
     def _table(self, batch, key, inv_freq, magnitude):
         table = batch.shared.get(key)
@@ -183,15 +189,23 @@ class PooledWindowAttention(Mixer):
                                 self.d, self.vd, self.pool)
         heads = rt.buffer("pooled_heads", (n, self.nh * self.vd))
         lens = batch.host_len
-        longest = int(lens.max()) if self.cores and lens is not None else 0
-        if longest >= self.LONG_ENTRY:
-            ops.pooled_attention_cores(q, kc, vc, kp, vp, batch.entry_start, batch.entry_len, batch.entry_past, longest,
-                                       view.block_tables, ptab, self.nh, self.nkv, self.d, self.vd, self.window, self.pool,
-                                       self.scale, out=heads, vtable=vtable, long_len=self.LONG_ENTRY)
-        if longest < self.LONG_ENTRY or int(lens.min()) < self.LONG_ENTRY:
-            ops.pooled_attention(q, kc, vc, kp, vp, batch.tok_seq, batch.positions, view.block_tables, ptab, self.nh, self.nkv,
-                                 self.d, self.vd, self.window, self.pool, self.scale, out=heads, vtable=vtable,
-                                 entry_len=batch.entry_len if longest >= self.LONG_ENTRY else None, long_len=self.LONG_ENTRY)
+        args = (self.nh, self.nkv, self.d, self.vd, self.window, self.pool, self.scale)
+        if not self.cores or lens is None:
+            ops.pooled_attention(q, kc, vc, kp, vp, batch.tok_seq, batch.positions, view.block_tables, ptab, *args, out=heads,
+                                 vtable=vtable)
+        else:
+            longest, shortest = int(lens.max()), int(lens.min())
+            if longest >= self.long_entry:
+                ops.pooled_attention_cores(q, kc, vc, kp, vp, batch.entry_start, batch.entry_len, batch.entry_past, longest,
+                                           view.block_tables, ptab, *args, out=heads, vtable=vtable, long_len=self.long_entry)
+            if shortest < self.long_entry:
+                max_keys = batch.plans[KEY_BOUND_PLANNER.key].sizes["max_keys"]
+                chunks, per = ops.pooled_attention_cores_cut(max_keys, self.window, self.pool, self.long_entry - 1, self.units,
+                                                             batch.num_entries * self.nkv)
+                ws = rt.buffer("pooled_chunks", (ops.pooled_attention_cores_workspace(n, self.nh, self.vd, chunks),), torch.float32)
+                ops.pooled_attention_cores(q, kc, vc, kp, vp, batch.entry_start, batch.entry_len, batch.entry_past, longest,
+                                           view.block_tables, ptab, *args, out=heads, vtable=vtable, long_len=self.long_entry,
+                                           chunks=chunks, chunk_blocks=per, workspace=ws, tok_seq=batch.tok_seq)
         if out is None:
             out = rt.buffer("pooled_out", (n, self.hidden))
         return ops.linear(heads, self.o, out=out)
