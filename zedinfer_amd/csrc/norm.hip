@@ -223,7 +223,7 @@ extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* d
 // w2 (1 + w2 with add_one): the norm that the next sublayer reads.  One workgroup a row; the row lies in LDS between
 // the passes.  The sums of squares are added in an order fixed by the row's width alone.
 template <typename TD, typename TW, typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 normed_add_norm_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD* __restrict__ y, int64_t ldy, int splits,
                        int64_t split_stride, const TW* __restrict__ w1, const TW* __restrict__ w2, int H, float eps,
                        float eps2, int add_one) {
@@ -234,7 +234,13 @@ normed_add_norm_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD
     float ss = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = zi_load(yr + i);
-        for (int s = 1; s < splits; ++s) v += zi_load(yr + s * split_stride + i);
+        int s = 1;
+        for (; s + 4 <= splits; s += 4) {      // four loads in flight; the additions keep their order
+            const float a = zi_load(yr + s * split_stride + i), b = zi_load(yr + (s + 1) * split_stride + i),
+                        c = zi_load(yr + (s + 2) * split_stride + i), d = zi_load(yr + (s + 3) * split_stride + i);
+            v += a; v += b; v += c; v += d;
+        }
+        for (; s < splits; ++s) v += zi_load(yr + s * split_stride + i);
         row_values[i] = v;
         ss += v * v;
     }
@@ -268,12 +274,15 @@ extern "C" int zi_normed_add_norm(void* out, int out_dt, float* resid, const voi
     ZI_REQUIRE(splits == 1 || y_dt == ZI_F32, "normed_add_norm: partial sums are float32");
     if (n == 0) return 0;
     const size_t lds = (size_t)hidden * sizeof(float);
+    // few rows: a thread walks few values (the sums of squares then add up in another order than with 256 threads, so
+    // the float32 path, whose results must not depend on the step's rows, keeps one size: its gains are float32)
+    const int threads = (n <= 64 && hidden > 512 && w_dt == ZI_BF16) ? 1024 : 256;
     ZI_DISPATCH_DTYPE(y_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, {
         if (!out || out_dt == ZI_F32)
-            normed_add_norm_kernel<TD, TW, float><<<n, 256, lds, stream>>>((float*)out, resid, (const TD*)y, ldy, splits,
+            normed_add_norm_kernel<TD, TW, float><<<n, threads, lds, stream>>>((float*)out, resid, (const TD*)y, ldy, splits,
                 split_stride, (const TW*)w1, (const TW*)w2, hidden, eps, eps2, add_one);
         else
-            normed_add_norm_kernel<TD, TW, zi_bf16><<<n, 256, lds, stream>>>((zi_bf16*)out, resid, (const TD*)y, ldy, splits,
+            normed_add_norm_kernel<TD, TW, zi_bf16><<<n, threads, lds, stream>>>((zi_bf16*)out, resid, (const TD*)y, ldy, splits,
                 split_stride, (const TW*)w1, (const TW*)w2, hidden, eps, eps2, add_one);
     }));
     return zi_check_launch("normed_add_norm");

@@ -24,6 +24,7 @@
 #define PA_MAX_D 512
 #define PA_ACC (PA_MAX_D / ZI_WAVE)
 #define PA_WAVES 4
+#define PB_ACC (2 * PA_MAX_D / ZI_WAVE)      // values of a key and a value a lane of the blocks' kernel sums
 
 // ---- norm, rotation, store ---------------------------------------------------------------------------------
 // One wavefront per (token, unit): units 0 .. nh-1 are the query heads, nh .. nh+nkv-1 the key/value heads.
@@ -132,21 +133,52 @@ pool_blocks_kernel(float* __restrict__ kpool, float* __restrict__ vpool, const T
     if (p + 1 < pool) return;
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
     const float inv = 1.f / (float)pool;
-    for (int i = lane; i < dim + vdim; i += ZI_WAVE) {
-        const bool key = i < dim;
-        float acc = 0.f;
-        for (int j = p - pool + 1; j <= p; ++j) {
-            const int pi = j / page_size;
+    // the block's rows in the cache, 64 positions at a time (a lane looks one up), then every lane walks them for its
+    // dims with the loads of eight positions in flight; the additions keep the order of the positions
+    __shared__ int64_t rows[ZI_WAVE];
+    float acc[PB_ACC];
+#pragma unroll
+    for (int a = 0; a < PB_ACC; ++a) acc[a] = 0.f;
+    const int width = dim + vdim;
+    for (int j0 = p - pool + 1; j0 <= p; j0 += ZI_WAVE) {
+        const int cnt = p - j0 + 1 < ZI_WAVE ? p - j0 + 1 : ZI_WAVE;
+        __syncthreads();
+        if (lane < cnt) {
+            const int j = j0 + lane, pi = j / page_size;
             const int page = pi < max_pages ? bt[pi] : -1;
-            if ((unsigned)page >= (unsigned)num_pages) {      // never scheduled: show it
-                acc = NAN;
-                continue;
-            }
-            const int64_t r = ((int64_t)page * page_size + j % page_size) * nkv + g;
-            acc += key ? zi_load(kcache + r * dim + i) : zi_load(vcache + r * vdim + (i - dim));
+            rows[lane] = (unsigned)page < (unsigned)num_pages ? ((int64_t)page * page_size + j % page_size) * nkv + g : -1;
         }
-        if (key) kpool[(ps * nkv + g) * dim + i] = acc * inv;
-        else vpool[(ps * nkv + g) * vdim + (i - dim)] = acc * inv;
+        __syncthreads();
+#pragma unroll
+        for (int a = 0; a < PB_ACC; ++a) {
+            const int i = lane + a * ZI_WAVE;
+            if (i >= width) break;
+            const bool key = i < dim;
+            const T* base = key ? kcache + i : vcache + (i - dim);
+            const int64_t stride = key ? dim : vdim;
+            int jj = 0;
+            for (; jj + 8 <= cnt; jj += 8) {
+                float x[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int64_t r = rows[jj + u];
+                    x[u] = r >= 0 ? zi_load(base + r * stride) : NAN;      // a hole is never scheduled: show it
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc[a] += x[u];
+            }
+            for (; jj < cnt; ++jj) {
+                const int64_t r = rows[jj];
+                acc[a] += r >= 0 ? zi_load(base + r * stride) : NAN;
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < PB_ACC; ++a) {
+        const int i = lane + a * ZI_WAVE;
+        if (i >= width) break;
+        if (i < dim) kpool[(ps * nkv + g) * dim + i] = acc[a] * inv;
+        else vpool[(ps * nkv + g) * vdim + (i - dim)] = acc[a] * inv;
     }
 }
 

@@ -34,7 +34,8 @@ ssm_prepare_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict
     const float* tail = state + (int64_t)entry_slot[e] * state_stride;
     const float* row = proj + (int64_t)t * ld;
     float* orow = out + (int64_t)t * ldo;
-    for (int c = threadIdx.x; c < C; c += SSM_THREADS) {
+    // (a token's channels are dealt out over the workgroups of its row of the launch)
+    for (int c = blockIdx.y * SSM_THREADS + threadIdx.x; c < C; c += gridDim.y * SSM_THREADS) {
         float acc = conv_b ? conv_b[c] : 0.f;
         for (int j = 0; j < taps; ++j) {
             const int li = local - (taps - 1) + j;
@@ -50,7 +51,7 @@ ssm_prepare_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict
             orow[C + c] = dt * x;
         }
     }
-    for (int h = threadIdx.x; h < heads; h += SSM_THREADS) {
+    for (int h = blockIdx.y * SSM_THREADS + threadIdx.x; h < heads; h += gridDim.y * SSM_THREADS) {
         const float dt = ssm_softplus(row[2 * inner + gn2 + h] + dt_bias[h]);
         orow[C + inner + h] = expf(-expf(a_log[h]) * dt);
     }
@@ -68,7 +69,11 @@ extern "C" int zi_ssm_prepare(float* out, int64_t ldo, const float* proj, int64_
     ZI_REQUIRE(ld >= width && ldo >= width, "ssm_prepare: a row is too short");
     ZI_REQUIRE(state_stride >= (int64_t)(taps - 1) * (inner + gn2), "ssm_prepare: the state row is too short");
     if (n == 0) return 0;
-    ssm_prepare_kernel<<<n, SSM_THREADS, 0, stream>>>(out, ldo, proj, ld, conv_w, conv_b, dt_bias, a_log, state,
+    // few tokens: a workgroup for every 256 channels of a token, so that a step of decoded tokens fills more of the chip
+    const int64_t C = inner + gn2;
+    int per_token = n >= 1024 ? 1 : (int)((C + SSM_THREADS - 1) / SSM_THREADS);
+    if (per_token > 64) per_token = 64;
+    ssm_prepare_kernel<<<dim3(n, per_token), SSM_THREADS, 0, stream>>>(out, ldo, proj, ld, conv_w, conv_b, dt_bias, a_log, state,
                                                       state_stride, tok_seq, entry_start, entry_slot, heads, vdim, gn2,
                                                       taps);
     return zi_check_launch("ssm_prepare");
