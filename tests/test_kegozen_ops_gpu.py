@@ -27,7 +27,7 @@ def _close(got, want, tol, what=""):
 
 
 @pytest.mark.parametrize("heads,vdim,N,G,taps,parts,cuts", [
-    (4, 16, 16, 2, 4, 2, [37]), (4, 16, 16, 2, 4, 2, [5, 1, 2, 20, 9]), (3, 24, 8, 1, 3, 1, [1, 1, 1, 30]),
+    (4, 16, 16, 2, 4, 2, [37]), (4, 16, 16, 2, 4, 2, [5, 1, 2, 20, 9]), (3, 24, 8, 1, 3, 1, [1, 1, 1, 30, 1, 1]), (2, 72, 40, 2, 4, 1, [1, 1, 1, 1, 5, 1]),
     (5, 20, 12, 5, 2, 5, [2, 2, 33]), (2, 64, 128, 1, 4, 1, [17, 3]), (6, 8, 40, 3, 1, 6, [11, 11])])
 def test_state_space_mechanism_whole_and_through_the_state(heads, vdim, N, G, taps, parts, cuts):
     from zedinfer_amd import ops
@@ -69,7 +69,8 @@ def test_state_space_mechanism_whole_and_through_the_state(heads, vdim, N, G, ta
             ops.conv_tail(state, pr[:, inner:inner + C], None, es, el, sl, taps)
         yy = torch.empty((n, inner), device=DEV)
         ops.linear_attention_grouped(prep[:, inner + gn:C], prep[:, inner:inner + gn], prep[:, C:C + inner], prep[:, C + inner:],
-                                     state[:, tail:], es, el, ep, sl, heads, heads // G, N, vdim, out=yy)
+                                     state[:, tail:], es, el, ep, sl, heads, heads // G, N, vdim, out=yy,
+                                     single_tokens=(n == 1 and at % 2 == 0))      # decoded tokens: either kernel
         ops.ssm_finish(yy, prep[:, :inner], pr[:, :inner], d(skip), d(gain), heads, vdim, parts, eps, out=got[at:at + n])
         at += n
     _close(got, want, 2e-4, "state space")

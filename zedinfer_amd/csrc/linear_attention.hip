@@ -228,17 +228,91 @@ linear_attention_kernel(float* __restrict__ out, int64_t ldo, const float* __res
     }
 }
 
+// The same recurrence for steps in which every entry brings ONE token: a workgroup per (entry, head) streams the
+// head's matrix through once, a wavefront a row at a time (64 consecutive columns a load: whole lines of memory),
+// the rows dealt out over the four wavefronts; the read-out's four partial sums are added in the wavefronts' order.
+// Its sums add up in another order than the kernel's above, so a token decoded alone and the same token inside a
+// portion agree within rounding, not to the bit.
+#define LA_STEP_MAX_DIM 512
+__global__ void __launch_bounds__(LA_WAVES* ZI_WAVE)
+linear_attention_step_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ q, const float* __restrict__ k,
+                             const float* __restrict__ v, int64_t ld, const float* __restrict__ decay, int64_t ld_decay,
+                             const float* __restrict__ head_decay, float* __restrict__ state, int64_t state_stride,
+                             const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
+                             const int32_t* __restrict__ entry_past, const int32_t* __restrict__ entry_slot, int dim,
+                             int vdim, int act, float qscale, int share, int decay_heads) {
+    __shared__ float ks[LA_STEP_MAX_DIM], qs[LA_STEP_MAX_DIM], as[LA_STEP_MAX_DIM];
+    __shared__ float part[LA_WAVES][ZI_WAVE];
+    const int head = blockIdx.x, e = blockIdx.y, tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    if (entry_len[e] != 1) return;
+    const int64_t t = entry_start[e];
+    const bool fresh = entry_past[e] == 0;
+    float* S = state + (int64_t)entry_slot[e] * state_stride + (int64_t)head * dim * vdim;
+    const float hd = head_decay ? head_decay[head] : 1.f;
+    const float at = (decay && decay_heads) ? decay[t * ld_decay + head] : hd;
+    for (int d = tid; d < dim; d += LA_WAVES * ZI_WAVE) {
+        float kk = k[t * ld + (int64_t)(head / share) * dim + d], qq = q[t * ld + (int64_t)(head / share) * dim + d];
+        if (act) {
+            kk = la_silu(kk);
+            qq = la_silu(qq);
+        }
+        ks[d] = kk;
+        qs[d] = qq * qscale;
+        as[d] = (decay && !decay_heads) ? decay[t * ld_decay + (int64_t)head * dim + d] : at;
+    }
+    __syncthreads();
+    for (int c0 = 0; c0 < vdim; c0 += ZI_WAVE) {
+        const int col = c0 + lane;
+        const bool live = col < vdim;
+        const int cc = live ? col : vdim - 1;
+        float vv = v[t * ld + (int64_t)head * vdim + cc];
+        if (act) vv = la_silu(vv);
+        float acc = 0.f;
+        int row = wave;
+        for (; row + 7 * LA_WAVES < dim; row += 8 * LA_WAVES) {      // eight rows' loads in flight
+            float sv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sv[u] = fresh ? 0.f : S[(int64_t)(row + u * LA_WAVES) * vdim + cc];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int r = row + u * LA_WAVES;
+                sv[u] = as[r] * sv[u] + ks[r] * vv;
+                acc += sv[u] * qs[r];
+                if (live) S[(int64_t)r * vdim + col] = sv[u];
+            }
+        }
+        for (; row < dim; row += LA_WAVES) {
+            float sv = fresh ? 0.f : S[(int64_t)row * vdim + cc];
+            sv = as[row] * sv + ks[row] * vv;
+            acc += sv * qs[row];
+            if (live) S[(int64_t)row * vdim + col] = sv;
+        }
+        part[wave][lane] = acc;
+        __syncthreads();
+        if (wave == 0 && live) {
+            float total = part[0][lane];
+#pragma unroll
+            for (int w = 1; w < LA_WAVES; ++w) total += part[w][lane];
+            out[t * ldo + (int64_t)head * vdim + col] = total;
+        }
+        __syncthreads();
+    }
+}
+
 // out [n][heads*vdim] float32 (row stride ldo).  q, k [n][(heads/share)*dim] and v [n][heads*vdim]: float32, one row
 // stride `ld` (columns of one projection); `share` heads in a row read the same q and k.  decay float32 (row stride
 // ld_decay): [n][heads*dim], or with `decay_heads` [n][heads], one factor a (token, head); or null; head_decay
 // [heads] or null (then 1).  state [slots][state_stride] float32, of which this layer's heads*dim*vdim floats start at
-// the pointer given.  act 1: SiLU of q, k and v as they are read.  q is multiplied by qscale.
+// the pointer given.  act 1: SiLU of q, k and v as they are read.  q is multiplied by qscale.  single_tokens: the
+// caller says that every entry brings one token (entries that do not are left alone): the kernel that streams a head's
+// matrix through once takes the step.
 extern "C" int zi_linear_attention_grouped(float* out, int64_t ldo, const float* q, const float* k, const float* v,
                                            int64_t ld, const float* decay, int64_t ld_decay, const float* head_decay,
                                            float* state, int64_t state_stride, const int32_t* entry_start,
                                            const int32_t* entry_len, const int32_t* entry_past,
                                            const int32_t* entry_slot, int entries, int heads, int dim, int vdim, int act,
-                                           float qscale, int share, int decay_heads, hipStream_t stream) {
+                                           float qscale, int share, int decay_heads, int single_tokens,
+                                           hipStream_t stream) {
     ZI_REQUIRE(entries >= 0 && entries <= 65535 && heads > 0 && heads <= 65535 && dim > 0 && vdim > 0,
                "linear_attention: bad sizes");
     ZI_REQUIRE(share > 0 && heads % share == 0, "linear_attention: %d heads do not share q and k in runs of %d", heads, share);
@@ -249,6 +323,12 @@ extern "C" int zi_linear_attention_grouped(float* out, int64_t ldo, const float*
     ZI_REQUIRE(!decay_heads || decay, "linear_attention: a decay a head and token must be given");
     ZI_REQUIRE(act == 0 || act == 1, "linear_attention: unknown activation %d", act);
     if (entries == 0) return 0;
+    if (single_tokens) {
+        linear_attention_step_kernel<<<dim3(heads, entries), LA_WAVES * ZI_WAVE, 0, stream>>>(
+            out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride, entry_start, entry_len, entry_past,
+            entry_slot, dim, vdim, act, qscale, share, decay_heads);
+        return zi_check_launch("linear_attention_step");
+    }
     const dim3 grid((vdim + LA_WCOLS - 1) / LA_WCOLS, heads, entries);
 #define ZI_LA(R, TC)                                                                                                 \
     if (decay)                                                                                                       \
@@ -275,7 +355,7 @@ extern "C" int zi_linear_attention(float* out, int64_t ldo, const float* q, cons
                                    int dim, int vdim, int act, float qscale, hipStream_t stream) {
     return zi_linear_attention_grouped(out, ldo, q, k, v, ld, decay, ld_decay, head_decay, state, state_stride,
                                        entry_start, entry_len, entry_past, entry_slot, entries, heads, dim, vdim, act,
-                                       qscale, 1, 0, stream);
+                                       qscale, 1, 0, 0, stream);
 }
 
 #define GATE_SIGMOID 0

@@ -256,7 +256,7 @@ int zi_rope_table_scaled(float* out, const int32_t* pos, const float* inv_freq, 
 int zi_linear_attention_grouped(float* out, int64_t ldo, const float* q, const float* k, const float* v, int64_t ld,
     const float* decay, int64_t ld_decay, const float* head_decay, float* state, int64_t state_stride, const int32_t*
     entry_start, const int32_t* entry_len, const int32_t* entry_past, const int32_t* entry_slot, int entries, int
-    heads, int dim, int vdim, int act, float qscale, int share, int decay_heads, hipStream_t stream);
+    heads, int dim, int vdim, int act, float qscale, int share, int decay_heads, int single_tokens, hipStream_t stream);
 // ssm.hip
 int zi_ssm_prepare(float* out, int64_t ldo, const float* proj, int64_t ld, int n, const float* conv_w, const float*
     conv_b, const float* dt_bias, const float* a_log, const float* state, int64_t state_stride, const int32_t*

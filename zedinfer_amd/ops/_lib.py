@@ -112,7 +112,7 @@ _PROTOTYPES = {
     "zi_attention_decode_biased": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P, F, P, I, I, P],
     "zi_moe_route_table": [P, P, P, P, I, I, I, I, P],
     "zi_rope_table_scaled": [P, P, P, I, I, F, P],
-    "zi_linear_attention_grouped": [P, L, P, P, P, L, P, L, P, P, L, P, P, P, P, I, I, I, I, I, F, I, I, P],
+    "zi_linear_attention_grouped": [P, L, P, P, P, L, P, L, P, P, L, P, P, P, P, I, I, I, I, I, F, I, I, I, P],
     "zi_ssm_prepare": [P, L, P, L, I, P, P, P, P, P, L, P, P, P, I, I, I, I, P],
     "zi_ssm_finish": [P, I, L, P, L, P, L, P, L, P, P, I, I, I, I, F, P],
     "zi_norm_rope_store": [P, I, L, P, P, P, L, I, L, P, P, F, P, I, P, P, L, I, I, I, I, I, P],

@@ -92,11 +92,12 @@ def ssm_finish(y: torch.Tensor, x: torch.Tensor, z: torch.Tensor, skip: torch.Te
 def linear_attention_grouped(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
                              entry_start: torch.Tensor, entry_len: torch.Tensor, entry_past: torch.Tensor,
                              entry_slot: torch.Tensor, heads: int, share: int, dim: int, vdim: int,
-                             out: torch.Tensor) -> torch.Tensor:
+                             out: torch.Tensor, single_tokens: bool = False) -> torch.Tensor:
     """Token by token over every entry, per head: S <- a_t S + k_t v_t^T, out_t = S^T q_t, where ``share`` heads in
     a row read the same q and k ([n, (heads/share)*dim]) and the decay a_t is one number a (token, head)
     ([n, heads]).  q, k, v and the decay are float32 column slices of ONE row; ``state`` [slots, >= heads*dim*vdim]
-    float32 (a column slice is fine)."""
+    float32 (a column slice is fine).  ``single_tokens``: every entry brings one token (the caller knows): the kernel
+    that streams every head's matrix through once takes the step; its sums differ from the other's by rounding."""
     _gpu("linear_attention_grouped", q, k, v, decay, state, entry_start, entry_len, entry_past, entry_slot, out)
     n = q.shape[0]
     if share <= 0 or heads % share:
@@ -117,7 +118,7 @@ def linear_attention_grouped(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
         _i32(t, "linear_attention_grouped entries", E)
     _lib.call("zi_linear_attention_grouped", _p(out), ldo, _p(q), _p(k), _p(v), max(ld, 1), _p(decay), max(ld, 1), None,
               _p(state), int(state.stride(0)), _p(entry_start), _p(entry_len), _p(entry_past), _p(entry_slot), E, heads,
-              dim, vdim, 0, 1.0, int(share), 1, _stream())
+              dim, vdim, 0, 1.0, int(share), 1, int(bool(single_tokens)), _stream())
     return out
 
 

@@ -94,7 +94,8 @@ class StateSpace(Mixer):
         y = rt.buffer("ssm_read", (n, inner), torch.float32)
         ops.linear_attention_grouped(prep[:, inner + gn:C], prep[:, inner:inner + gn], prep[:, C:C + inner],
                                      prep[:, C + inner:], state[:, self.tail:], batch.entry_start, batch.entry_len,
-                                     batch.entry_past, batch.entry_slot, self.nh, self.nh // self.G, self.N, self.vd, out=y)
+                                     batch.entry_past, batch.entry_slot, self.nh, self.nh // self.G, self.N, self.vd, out=y,
+                                     single_tokens=bool(batch.single_tokens))
         g = rt.buffer("ssm_gated", (n, inner))
         ops.ssm_finish(y, prep[:, :inner], proj[:, :inner], self.skip, self.norm, self.nh, self.vd, self.parts, self.eps, out=g)
         if out is None:
