@@ -118,67 +118,80 @@ extern "C" int zi_norm_rope_store(void* q_out, int dt, int64_t ldq, void* kcache
 }
 
 // ---- the blocks' means -------------------------------------------------------------------------------------
-// One workgroup per (token, key/value head); a token whose position does not end a block has pool slot -1.
+// One workgroup of four wavefronts per (token, key/value head); a token whose position does not end a block has pool
+// slot -1 and its workgroup leaves at once.  The block's rows in the cache are looked up 64 positions at a time (a
+// thread each); the wavefronts take the positions in turn (wavefront w: w, w + 4, ...), a lane the dims lane, lane +
+// 64, ..., with the loads of eight positions in flight and no load under a branch; the four partial sums are added in
+// the wavefronts' order.  The order of the additions depends on the block's length alone.
 template <typename T>
-__global__ void __launch_bounds__(ZI_WAVE)
+__global__ void __launch_bounds__(PA_WAVES* ZI_WAVE)
 pool_blocks_kernel(float* __restrict__ kpool, float* __restrict__ vpool, const T* __restrict__ kcache,
                    const T* __restrict__ vcache, const int32_t* __restrict__ pool_slots, int64_t pool_rows,
                    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                    const int32_t* __restrict__ block_tables, int max_pages, int num_pages, int page_size, int nkv,
                    int dim, int vdim, int pool) {
-    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+    __shared__ int64_t rows[ZI_WAVE];
+    __shared__ float parts[PA_WAVES][2 * PA_MAX_D];
+    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
     const int64_t ps = pool_slots[t];
     if (ps < 0 || ps >= pool_rows) return;
     const int p = tok_pos[t];
     if (p + 1 < pool) return;
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
     const float inv = 1.f / (float)pool;
-    // the block's rows in the cache, 64 positions at a time (a lane looks one up), then every lane walks them for its
-    // dims with the loads of eight positions in flight; the additions keep the order of the positions
-    __shared__ int64_t rows[ZI_WAVE];
     float acc[PB_ACC];
 #pragma unroll
     for (int a = 0; a < PB_ACC; ++a) acc[a] = 0.f;
     const int width = dim + vdim;
+    bool hole = false;      // a position without a page is never scheduled: it shows as NaN
     for (int j0 = p - pool + 1; j0 <= p; j0 += ZI_WAVE) {
         const int cnt = p - j0 + 1 < ZI_WAVE ? p - j0 + 1 : ZI_WAVE;
         __syncthreads();
-        if (lane < cnt) {
-            const int j = j0 + lane, pi = j / page_size;
+        if (tid < cnt) {
+            const int j = j0 + tid, pi = j / page_size;
             const int page = pi < max_pages ? bt[pi] : -1;
-            rows[lane] = (unsigned)page < (unsigned)num_pages ? ((int64_t)page * page_size + j % page_size) * nkv + g : -1;
+            rows[tid] = (unsigned)page < (unsigned)num_pages ? ((int64_t)page * page_size + j % page_size) * nkv + g : -1;
         }
         __syncthreads();
 #pragma unroll
         for (int a = 0; a < PB_ACC; ++a) {
             const int i = lane + a * ZI_WAVE;
-            if (i >= width) break;
-            const bool key = i < dim;
-            const T* base = key ? kcache + i : vcache + (i - dim);
-            const int64_t stride = key ? dim : vdim;
-            int jj = 0;
-            for (; jj + 8 <= cnt; jj += 8) {
-                float x[8];
+            if (i < width) {
+                const bool key = i < dim;
+                const T* base = key ? kcache + i : vcache + (i - dim);
+                const int64_t stride = key ? dim : vdim;
+                int jj = wave;
+                for (; jj + 7 * PA_WAVES < cnt; jj += 8 * PA_WAVES) {
+                    float x[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int64_t r = rows[jj + u];
-                    x[u] = r >= 0 ? zi_load(base + r * stride) : NAN;      // a hole is never scheduled: show it
+                    for (int u = 0; u < 8; ++u) {
+                        const int64_t r = rows[jj + u * PA_WAVES];
+                        hole |= r < 0;
+                        x[u] = zi_load(base + (r < 0 ? 0 : r) * stride);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc[a] += x[u];
                 }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) acc[a] += x[u];
-            }
-            for (; jj < cnt; ++jj) {
-                const int64_t r = rows[jj];
-                acc[a] += r >= 0 ? zi_load(base + r * stride) : NAN;
+                for (; jj < cnt; jj += PA_WAVES) {
+                    const int64_t r = rows[jj];
+                    hole |= r < 0;
+                    acc[a] += zi_load(base + (r < 0 ? 0 : r) * stride);
+                }
             }
         }
     }
 #pragma unroll
     for (int a = 0; a < PB_ACC; ++a) {
         const int i = lane + a * ZI_WAVE;
-        if (i >= width) break;
-        if (i < dim) kpool[(ps * nkv + g) * dim + i] = acc[a] * inv;
-        else vpool[(ps * nkv + g) * vdim + (i - dim)] = acc[a] * inv;
+        if (i < width) parts[wave][i] = hole ? NAN : acc[a];
+    }
+    __syncthreads();
+    for (int i = tid; i < width; i += PA_WAVES * ZI_WAVE) {
+        float total = parts[0][i];
+#pragma unroll
+        for (int w = 1; w < PA_WAVES; ++w) total += parts[w][i];
+        if (i < dim) kpool[(ps * nkv + g) * dim + i] = total * inv;
+        else vpool[(ps * nkv + g) * vdim + (i - dim)] = total * inv;
     }
 }
 
@@ -190,7 +203,7 @@ extern "C" int zi_pool_blocks(float* kpool, float* vpool, int64_t pool_rows, con
                    num_pages > 0 && pool_rows > 0, "pool_blocks: bad sizes");
     if (n == 0) return 0;
     ZI_DISPATCH_DTYPE(dt, T, {
-        pool_blocks_kernel<T><<<dim3(n, nkv), ZI_WAVE, 0, stream>>>(kpool, vpool, (const T*)kcache, (const T*)vcache,
+        pool_blocks_kernel<T><<<dim3(n, nkv), PA_WAVES * ZI_WAVE, 0, stream>>>(kpool, vpool, (const T*)kcache, (const T*)vcache,
                                                                     pool_slots, pool_rows, tok_seq, tok_pos, block_tables,
                                                                     max_pages, num_pages, page_size, nkv, dim, vdim, pool);
     });

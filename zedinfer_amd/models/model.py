@@ -84,6 +84,14 @@ class DecoderModel:
         # what a schedule step does to the stream before its layer runs
         self.enters = [(_build(STREAM_STEPS, st.enter, weights, rt) if st.enter is not None else None) for st in fc.schedule]
         self.parts += [e for e in self.enters if e is not None]
+        # What a block may know of the step after it: the norm that the next block runs first, so that an arrangement
+        # whose last launch is a norm of its own can make the next one in the same launch (None: the last step, a
+        # stream step in between, or a block without such a norm).
+        self.next_input_norms = []
+        for i, st in enumerate(fc.schedule):
+            nxt = fc.schedule[i + 1] if i + 1 < len(fc.schedule) else None
+            ok = nxt is not None and nxt.enter is None
+            self.next_input_norms.append(getattr(self.blocks[nxt.layer], "norm_in", None) if ok else None)
         self.keeps_embedded = any(getattr(e, "needs_embedded", False) for e in self.enters if e is not None)
         self.final_norm = _build(NORMS, fc.final_norm, weights, rt)
         self.lm_head = _build(HEADS, fc.lm_head, weights, rt)
@@ -196,9 +204,11 @@ class DecoderModel:
         if self.keeps_embedded:
             embedded = ops.convert(resid, self.rt.buffer("embedded", tuple(resid.shape), torch.float32))
         delta = None
-        for st, mem, enter in zip(self.fc.schedule, memories, self.enters):
+        for st, mem, enter, next_norm in zip(self.fc.schedule, memories, self.enters, self.next_input_norms):
             if enter is not None:
                 delta = enter.forward(resid, delta, embedded)
+            if shared is not None:
+                shared["next_input_norm"] = next_norm
             delta = self.blocks[st.layer].forward(resid, delta, batch, mem)
         if batch.num_logit_rows == 0:
             if delta is not None:

@@ -138,12 +138,15 @@ class SandwichBlock(Block):
     norm after each sublayer.  The norms on the outputs must offer ``add_normed`` (the RMS norm does): the output's
     norm, the addition into the float32 stream and the norm that the feed-forward reads are one launch.  Nothing is
     left pending: the stream is whole when the block returns.  The feed-forward may be the kind "none" (its two
-    norms are then the kind "none" too)."""
+    norms are then the kind "none" too).  When the model says which norm the next block runs first
+    (``batch.shared["next_input_norm"]``) and that norm is of the same kind, the block's last launch makes it too and
+    hands the rows on (``batch.shared[SHARED]``: the norm and its rows), which the next block of the kind takes up."""
 
     graph_safe = True
     tape_safe = True
 
     norm_names = ("input", "mixer_out", "ff_in", "ff_out")
+    SHARED = "sandwich_block.normed_input"
 
     def __init__(self, norms, mixer, feed_forward, rt: Runtime):
         self.norm_in, self.norm_mixer_out = norms["input"], norms["mixer_out"]
@@ -154,13 +157,31 @@ class SandwichBlock(Block):
         self.rt = rt
 
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, memory: LayerMemory):
-        x = self.norm_in.add_forward(resid, delta) if delta is not None else self.norm_in.forward(resid)
+        shared = getattr(batch, "shared", None)
+        ready = shared.pop(self.SHARED, None) if shared is not None else None
+        if delta is not None:
+            x = self.norm_in.add_forward(resid, delta)
+        elif ready is not None and ready[0] is self.norm_in:
+            x = ready[1]                      # the block before made this norm in its last launch
+        else:
+            x = self.norm_in.forward(resid)
+        then = shared.get("next_input_norm") if shared is not None else None
+        if then is not None and not self._same_kind(then):
+            then = None
         a = self.mixer.forward(x, batch, memory)
         if not self.has_ff:
-            self.norm_mixer_out.add_normed(resid, a)
-            return None
-        y = self.norm_mixer_out.add_normed(resid, a, then=self.norm_ff_in)
-        kw = {"batch": batch} if self.feed_forward.reads_batch else {}
-        f = self.feed_forward.forward(y, **kw)
-        self.norm_ff_out.add_normed(resid, f)
+            out = self.norm_mixer_out.add_normed(resid, a, then=then)
+        else:
+            y = self.norm_mixer_out.add_normed(resid, a, then=self.norm_ff_in)
+            kw = {"batch": batch} if self.feed_forward.reads_batch else {}
+            f = self.feed_forward.forward(y, **kw)
+            out = self.norm_ff_out.add_normed(resid, f, then=then)
+        if then is not None:
+            shared[self.SHARED] = (then, out)
         return None
+
+    def _same_kind(self, norm) -> bool:
+        last = self.norm_ff_out if self.has_ff else self.norm_mixer_out
+        return (type(norm) is type(last) and getattr(norm, "add_one", None) == getattr(last, "add_one", None)
+                and getattr(norm, "weight", None) is not None and norm.weight.dtype == last.weight.dtype
+                and getattr(norm, "out_dtype", None) is None)

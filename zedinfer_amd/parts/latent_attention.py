@@ -154,5 +154,8 @@ class LatentAttention(Mixer):
                                  self.window, out=o)
         heads = ops.latent_value(o, self.uv, self.vdim, out=rt.buffer("latent_heads", (n, self.nh * self.vdim)))
         if out is None:
+            if ops.linear_sums_supported(heads, self.o):      # few rows: the partial sums go to the norm that follows
+                S = ops.linear_splits(n, self.hidden, self.nh * self.vdim)
+                return ops.linear_sums(heads, self.o, out=rt.buffer("latent_out_sums", (S, n, self.hidden), torch.float32))
             out = rt.buffer("latent_out", (n, self.hidden))
         return ops.linear(heads, self.o, out=out)

@@ -173,10 +173,15 @@ class PooledWindowAttention(Mixer):
         kc, vc = memory.tensors["k"], memory.tensors["v"]
         table = self._table(batch, self.table_key, self.inv_freq, self.magnitude) if self.rot else None
         vtable = self._table(batch, self.vtable_key, self.v_inv_freq, 1.0) if self.rotate_values else None
-        full = ops.linear(x, self.qkv, out=rt.buffer("pooled_qkv", (n, self.qkv.shape[0]), torch.float32))
+        if ops.linear_sums_supported(x, self.qkv) and self.qkv.shape[0] == self.width:
+            # few rows: the kernel that norms and stores adds the product's partial sums itself
+            S = ops.linear_splits(n, self.width, self.hidden)
+            proj = ops.linear_sums(x, self.qkv, out=rt.buffer("pooled_qkv_sums", (S, n, self.width), torch.float32))
+        else:
+            proj = ops.linear(x, self.qkv, out=rt.buffer("pooled_qkv", (n, self.qkv.shape[0]), torch.float32))[:, :self.width]
         q = rt.buffer("pooled_q", (n, self.nh * self.d))
         writes = memory.writes
-        ops.norm_rope_store(full[:, :self.width], self.q_gain, self.k_gain, self.eps, table, vtable,
+        ops.norm_rope_store(proj, self.q_gain, self.k_gain, self.eps, table, vtable,
                             view.slots if writes else None, kc if writes else None, vc if writes else None,
                             self.nh, self.nkv, self.d, self.vd, q_out=q)
         blocks = memory.sides.get("blocks") if self.pool > 0 else None
@@ -207,5 +212,8 @@ class PooledWindowAttention(Mixer):
                                            view.block_tables, ptab, *args, out=heads, vtable=vtable, long_len=self.long_entry,
                                            chunks=chunks, chunk_blocks=per, workspace=ws, tok_seq=batch.tok_seq)
         if out is None:
+            if ops.linear_sums_supported(heads, self.o):      # few rows: the partial sums go to the norm that follows
+                S = ops.linear_splits(n, self.hidden, self.nh * self.vd)
+                return ops.linear_sums(heads, self.o, out=rt.buffer("pooled_out_sums", (S, n, self.hidden), torch.float32))
             out = rt.buffer("pooled_out", (n, self.hidden))
         return ops.linear(heads, self.o, out=out)

@@ -99,5 +99,8 @@ class StateSpace(Mixer):
         g = rt.buffer("ssm_gated", (n, inner))
         ops.ssm_finish(y, prep[:, :inner], proj[:, :inner], self.skip, self.norm, self.nh, self.vd, self.parts, self.eps, out=g)
         if out is None:
+            if ops.linear_sums_supported(g, self.o):      # few rows: the partial sums go to the norm that follows
+                S = ops.linear_splits(n, self.hidden, inner)
+                return ops.linear_sums(g, self.o, out=rt.buffer("ssm_out_sums", (S, n, self.hidden), torch.float32))
             out = rt.buffer("ssm_out", (n, self.hidden))
         return ops.linear(g, self.o, out=out)
