@@ -139,6 +139,68 @@ pool_blocks_kernel(float* __restrict__ kpool, float* __restrict__ vpool, const T
     if (p + 1 < pool) return;
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
     const float inv = 1.f / (float)pool;
+    if constexpr (sizeof(T) == 2) {
+        // bfloat16 rows whose widths are multiples of 8: a thread loads 16 bytes (8 dims) of a position at a time, so a
+        // block of 64 positions is two loads a thread, all in flight together; the positions are dealt out over the
+        // threads that share a piece of 8 dims (thread: piece tid % pieces, positions tid / pieces, + groups, ...), the
+        // groups' partial sums are added in the groups' order
+        const int pieces = (dim + vdim) / 8;
+        if (dim % 8 == 0 && vdim % 8 == 0 && pieces <= PA_WAVES * ZI_WAVE && ((uintptr_t)kcache % 16) == 0 &&
+            ((uintptr_t)vcache % 16) == 0) {
+            const int groups = PA_WAVES * ZI_WAVE / pieces;      // at most 2 * PA_MAX_D / 8 = 128 pieces: at least 2 groups
+            const int piece = tid % pieces, grp = tid / pieces;
+            const bool works = grp < groups;
+            const bool key = piece * 8 < dim;
+            const T* base = key ? kcache + piece * 8 : vcache + (piece * 8 - dim);
+            const int64_t stride = key ? dim : vdim;
+            float a8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            bool hole = false;
+            for (int j0 = p - pool + 1; j0 <= p; j0 += ZI_WAVE) {
+                const int cnt = p - j0 + 1 < ZI_WAVE ? p - j0 + 1 : ZI_WAVE;
+                __syncthreads();
+                if (tid < cnt) {
+                    const int j = j0 + tid, pi = j / page_size;
+                    const int page = pi < max_pages ? bt[pi] : -1;
+                    rows[tid] = (unsigned)page < (unsigned)num_pages ? ((int64_t)page * page_size + j % page_size) * nkv + g : -1;
+                }
+                __syncthreads();
+                if (works) {
+                    for (int jj = grp; jj < cnt; jj += 4 * groups) {
+                        uint4 x[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int at = jj + u * groups;
+                            const int64_t r = rows[at < cnt ? at : jj];
+                            hole |= r < 0;
+                            x[u] = *reinterpret_cast<const uint4*>(base + (r < 0 ? 0 : r) * stride);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            if (jj + u * groups >= cnt) continue;
+                            a8[0] += __uint_as_float(x[u].x << 16); a8[1] += __uint_as_float(x[u].x & 0xffff0000u);
+                            a8[2] += __uint_as_float(x[u].y << 16); a8[3] += __uint_as_float(x[u].y & 0xffff0000u);
+                            a8[4] += __uint_as_float(x[u].z << 16); a8[5] += __uint_as_float(x[u].z & 0xffff0000u);
+                            a8[6] += __uint_as_float(x[u].w << 16); a8[7] += __uint_as_float(x[u].w & 0xffff0000u);
+                        }
+                    }
+                }
+            }
+            // parts as [group][dim]: groups * (dim + vdim) <= 256 * 8 floats
+            float* flat = &parts[0][0];
+            if (works) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) flat[(int64_t)grp * pieces * 8 + piece * 8 + i] = hole ? NAN : a8[i];
+            }
+            __syncthreads();
+            for (int i = tid; i < pieces * 8; i += PA_WAVES * ZI_WAVE) {
+                float total = flat[i];
+                for (int w = 1; w < groups; ++w) total += flat[(int64_t)w * pieces * 8 + i];
+                if (i < dim) kpool[(ps * nkv + g) * dim + i] = total * inv;
+                else vpool[(ps * nkv + g) * vdim + (i - dim)] = total * inv;
+            }
+            return;
+        }
+    }
     float acc[PB_ACC];
 #pragma unroll
     for (int a = 0; a < PB_ACC; ++a) acc[a] = 0.f;
