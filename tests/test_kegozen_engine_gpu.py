@@ -261,3 +261,32 @@ def test_the_replay_tool_runs_a_model_of_the_design(tmp_path):
     steps = traces.mixed(requests, max_live=4, seed=11)
     out = traces.run_tool(folder, "float32", steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
     assert _check(steps, out, ref, "float32", "replay tool") == sum(len(t) for t in requests.values())
+
+
+def test_command_lines_take_a_model_of_the_design(tmp_path):
+    """random_model writes a folder from the design's config.json (the engine's own random weights: gains of zero
+    around one, zero biases), ping generates from it what the plain implementation generates, batch_bench runs its
+    scheduler over it."""
+    import subprocess
+    import sys
+    root = traces.ROOT
+    env = dict(os.environ, PYTHONPATH=root)
+    run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300,  # noqa: E731
+                                    cwd=str(tmp_path))
+    (tmp_path / "cfg").mkdir()
+    with open(tmp_path / "cfg" / "config.json", "w") as f:
+        json.dump(models.ODD, f)
+    folder = str(tmp_path / "made")
+    r = run(os.path.join(root, "bin", "random_model"), str(tmp_path / "cfg"), folder, "--seed", "5", "--dtype", "float32", "--std", "0.1", "--noisy-norms")
+    assert r.returncode == 0, r.stderr + r.stdout
+    ref_model = plain.PlainKegozen.from_folder(folder)
+    assert set(ref_model.w) == set(models.tensor_shapes(models.ODD))
+    prompt = traces.random_tokens(models.ODD["vocab"], 27, seed=3)
+    r = run(os.path.join(root, "bin", "ping"), folder, "--dtype", "fp32", "--prompt-ids", ",".join(map(str, prompt)),
+            "--max-new-tokens", "6", "--ignore-eos", "--num-kv-blocks", "32", "--kv-block-size", "8", "--no-log-to-console")
+    assert r.returncode == 0, r.stderr
+    want = ref_model.greedy_generate(prompt, 6)
+    assert "output_ids: " + ",".join(map(str, want)) in r.stdout, r.stdout
+    r = run(os.path.join(root, "bin", "batch_bench"), str(tmp_path / "cfg"), "-b", "3", "-p", "20", "-d", "6", "--num-kv-blocks",
+            "64", "--kv-block-size", "8", "--random-weights", "--seed", "4", "--no-log-to-console")
+    assert r.returncode == 0 and "18 tokens generated" in r.stdout, r.stderr + r.stdout
